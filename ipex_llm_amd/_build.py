@@ -81,6 +81,9 @@ def _cmd(src: str, obj: str):
             # some of them (profiles/gemv5_xm_forms_r6.txt)
             if os.path.basename(src) == "gemv_int4_xm.hip":
                 extra = ["-fno-slp-vectorize"]
+        if os.path.basename(src) == "seqmix.hip":
+            # f32-exact kernels: no packed-f32 instruction forms
+            extra = ["-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
         return [HIPCC, f"--offload-arch={ARCH}", "-Wno-pass-failed", *extra, *common, "-c", src, "-o", obj]
     if "/cpu/" in src:
         return ["g++", *common, "-fopenmp", "-march=x86-64-v3", "-c", src, "-o", obj]
@@ -90,18 +93,41 @@ def _cmd(src: str, obj: str):
             "-I", tinc, "-I", tapi, "-I", pyinc, "-c", src, "-o", obj]
 
 
-def sources():
+# partial libraries: the translation units one model kind needs, linked alone
+TARGETS = {
+    # hybrid decoders: sequence-mixing kernels + their bindings + the serving scheduler
+    "seqmix": ["hip/seqmix.hip", "torch/ops_seqmix.cpp", "runtime/scheduler.cpp"],
+}
+
+
+def _target_lib(target):
+    return LIB if not target else os.path.join(PKG, f"_C_{target}.so")
+
+
+def sources(target=None):
+    if target:
+        return [os.path.join(CSRC, *rel.split("/")) for rel in TARGETS[target]]
     return sorted(glob.glob(os.path.join(CSRC, "hip", "*.hip")) +
                   glob.glob(os.path.join(CSRC, "cpu", "*.cpp")) +
                   glob.glob(os.path.join(CSRC, "torch", "*.cpp")) +
                   glob.glob(os.path.join(CSRC, "runtime", "*.cpp")))
 
 
-def build(verbose: bool = False, jobs: int | None = None, force: bool = False) -> str:
+def needs_build(target=None) -> bool:
+    """True when the target's library is missing or older than one of its sources / headers."""
+    lib = _target_lib(target)
+    if not os.path.exists(lib):
+        return True
+    newest = max([os.path.getmtime(s) for s in sources(target)] + [_headers_mtime()])
+    return os.path.getmtime(lib) < newest
+
+
+def build(verbose: bool = False, jobs: int | None = None, force: bool = False, target: str | None = None) -> str:
     os.makedirs(OBJ, exist_ok=True)
     hdr = _headers_mtime()
     todo, objs = [], []
-    for src in sources():
+    LIB = _target_lib(target)
+    for src in sources(target):
         rel = os.path.relpath(src, CSRC).replace(os.sep, "_")
         obj = os.path.join(OBJ, rel + ".o")
         objs.append(obj)
@@ -143,4 +169,5 @@ def build(verbose: bool = False, jobs: int | None = None, force: bool = False) -
 
 
 if __name__ == "__main__":
-    build(verbose=True, force="--force" in sys.argv)
+    _t = next((a.split("=", 1)[1] for a in sys.argv if a.startswith("--target=")), None)
+    build(verbose=True, force="--force" in sys.argv, target=_t)

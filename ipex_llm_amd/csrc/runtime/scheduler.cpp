@@ -56,6 +56,8 @@ struct Seq {
   int64_t preemptions = 0;
   std::vector<int64_t> blocks;
   std::vector<int64_t> toks;  // prompt + generated ids (prefix caching only)
+  int64_t slot = -1;          // recurrent-state slot (set_state_slots), -1: none
+  bool external = false;      // opened with open(): fed from outside, grows with extend()
   int64_t nhashed = 0;        // leading full blocks already hashed / registered
   uint64_t last_hash = kSeed; // chain hash after nhashed blocks
 };
@@ -185,6 +187,119 @@ class Scheduler : public torch::CustomClassHolder {
     return out;
   }
 
+  // ---- recurrent-state slots (hybrid models): every running sequence holds
+  // one of n slots from admission to finish / preemption
+  void set_state_slots(int64_t n) {
+    TORCH_CHECK(n > 0, "Scheduler: bad slot count");
+    TORCH_CHECK(running_.empty(), "Scheduler: set_state_slots with running sequences");
+    slots_on_ = true;
+    free_slots_.clear();
+    for (int64_t i = n - 1; i >= 0; i--) free_slots_.push_back(i);
+  }
+  int64_t slot(int64_t id) { return get(id).slot; }
+  int64_t num_free_slots() { return slots_on_ ? (int64_t)free_slots_.size() : -1; }
+
+  // ---- externally fed sequence: its tokens arrive step by step and its final
+  // length is unknown, so blocks are taken as it grows (extend) instead of at
+  // admission.  It never waits and is never preempted by schedule*().
+  void open(int64_t id) {
+    TORCH_CHECK(!seqs_.count(id), "Scheduler: duplicate request id ", id);
+    TORCH_CHECK((int64_t)running_.size() < max_batch_, "Scheduler: batch is full");
+    Seq s;
+    s.id = id;
+    s.state = RUNNING;
+    s.external = true;
+    s.admitted = ++admit_counter_;
+    if (slots_on_) {
+      TORCH_CHECK(!free_slots_.empty(), "Scheduler: no free state slot");
+      s.slot = free_slots_.back();
+      free_slots_.pop_back();
+    }
+    seqs_[id] = s;
+    running_.push_back(id);
+  }
+  // room for n more tokens after the cached ones
+  void extend(int64_t id, int64_t n) {
+    Seq& s = get(id);
+    TORCH_CHECK(s.state == RUNNING && n >= 0, "Scheduler: extend on a sequence that is not running");
+    const int64_t need = blocks_for(s.cached + n);
+    TORCH_CHECK(need - (int64_t)s.blocks.size() <= available(), "Scheduler: KV pool exhausted (need ",
+                need - (int64_t)s.blocks.size(), " blocks, ", available(), " free)");
+    while ((int64_t)s.blocks.size() < need) s.blocks.push_back(pop_free());
+    if (s.cached + n > s.context) s.context = s.cached + n;
+  }
+
+  // ---- mixed steps (models whose forward takes ragged batches): every
+  // running sequence brings min(context - cached, budget left) tokens -- one
+  // for a decoding sequence, a portion of its prompt for one still prefilling
+  // -- and waiting requests are admitted behind them under the same budget.
+  // -> [id, n, id, n, ..., -1, preempted ids..., -1, failed ids...]
+  std::vector<int64_t> schedule_mixed() {
+    std::vector<int64_t> work, preempted, failed;
+    int64_t budget = max_prefill_;
+    std::vector<int64_t> run(running_.begin(), running_.end());
+    for (size_t i = 0; i < run.size(); i++) {
+      Seq& s = seqs_[run[i]];
+      if (s.state != RUNNING || s.external) continue;
+      int64_t n = std::min(s.context - s.cached, budget);
+      if (n <= 0) continue;
+      bool gone = false;
+      while (s.cached + n > (int64_t)s.blocks.size() * bs_) {
+        if (available() > 0) {
+          s.blocks.push_back(pop_free());
+          continue;
+        }
+        int64_t victim = -1, best = -1;
+        for (int64_t r : running_) {
+          const Seq& c = seqs_[r];
+          if (c.state == RUNNING && !c.external && c.admitted > best) { best = c.admitted; victim = r; }
+        }
+        TORCH_CHECK(victim >= 0, "Scheduler: KV pool exhausted");
+        // a victim already given work this step loses it
+        for (size_t w = 0; w + 1 < work.size(); w += 2)
+          if (work[w] == victim) { budget += work[w + 1]; work.erase(work.begin() + w, work.begin() + w + 2); break; }
+        preempt(victim);
+        preempted.push_back(victim);
+        if (victim == s.id) { gone = true; break; }
+      }
+      if (gone) continue;
+      work.push_back(s.id);
+      work.push_back(n);
+      budget -= n;
+    }
+    while (!waiting_.empty() && (int64_t)running_.size() < max_batch_ && budget > 0) {
+      Seq& s = seqs_[waiting_.front()];
+      const int64_t need = blocks_for(s.context + 1);
+      if (need > total_) {
+        s.state = FAILED;
+        failed.push_back(s.id);
+        waiting_.pop_front();
+        continue;
+      }
+      if (need > available() || (slots_on_ && free_slots_.empty())) break;
+      waiting_.pop_front();
+      for (int64_t i = 0; i < need; i++) s.blocks.push_back(pop_free());
+      if (slots_on_) {
+        s.slot = free_slots_.back();
+        free_slots_.pop_back();
+      }
+      s.state = RUNNING;
+      s.cached = 0;
+      s.admitted = ++admit_counter_;
+      running_.push_back(s.id);
+      const int64_t n = std::min(s.context, budget);
+      work.push_back(s.id);
+      work.push_back(n);
+      budget -= n;
+    }
+    std::vector<int64_t> out(work);
+    out.push_back(-1);
+    out.insert(out.end(), preempted.begin(), preempted.end());
+    out.push_back(-1);
+    out.insert(out.end(), failed.begin(), failed.end());
+    return out;
+  }
+
   // n new tokens of sequence id now have K/V in the cache
   void advance(int64_t id, int64_t n) {
     Seq& s = get(id);
@@ -260,6 +375,10 @@ class Scheduler : public torch::CustomClassHolder {
     s.blocks.clear();
     s.nhashed = 0;
     s.last_hash = kSeed;
+    if (s.slot >= 0) {
+      free_slots_.push_back(s.slot);
+      s.slot = -1;
+    }
   }
   // longest chain of cached full blocks covering the context minus its last token
   void match_prefix(const Seq& s, std::vector<int64_t>& hit, uint64_t& chain) {
@@ -316,6 +435,8 @@ class Scheduler : public torch::CustomClassHolder {
   std::vector<int64_t> etick_;                        // LRU tick of an idle cached block (-1: not idle)
   std::set<std::pair<int64_t, int64_t>> evict_;       // idle cached blocks, oldest first
   int64_t tick_ = 0, hit_tokens_ = 0;
+  bool slots_on_ = false;
+  std::vector<int64_t> free_slots_;
   std::deque<int64_t> waiting_;
   std::vector<int64_t> running_;
   std::unordered_map<int64_t, Seq> seqs_;
@@ -343,5 +464,11 @@ TORCH_LIBRARY_FRAGMENT(ipex_llm_amd, m) {
       .def("num_free_blocks", &Scheduler::num_free_blocks)
       .def("num_waiting", &Scheduler::num_waiting)
       .def("num_running", &Scheduler::num_running)
-      .def("block_size", &Scheduler::block_size);
+      .def("block_size", &Scheduler::block_size)
+      .def("set_state_slots", &Scheduler::set_state_slots)
+      .def("slot", &Scheduler::slot)
+      .def("num_free_slots", &Scheduler::num_free_slots)
+      .def("open", &Scheduler::open)
+      .def("extend", &Scheduler::extend)
+      .def("schedule_mixed", &Scheduler::schedule_mixed);
 }

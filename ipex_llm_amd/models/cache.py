@@ -32,6 +32,71 @@ class BlockAllocator:
         self.free.extend(reversed(blocks))
 
 
+class SlotAllocator:
+    """Free list of recurrent-state slots (one per live sequence).  A slot's
+    content is never cleared on release: a sequence whose first position is 0
+    starts from the zero state inside the scan kernels, whatever the slot held."""
+
+    def __init__(self, num_slots: int):
+        self.free: List[int] = list(range(num_slots - 1, -1, -1))
+
+    def alloc(self) -> int:
+        if not self.free:
+            raise RuntimeError("recurrent-state pool exhausted: no free slot")
+        return self.free.pop()
+
+    def release(self, slot: int):
+        self.free.append(slot)
+
+
+class HybridCache:
+    """Cache of a model whose layers mix paged attention rows and recurrent
+    state (models/hybrid.py).
+
+    ``layer_specs[i]`` is ``("rows", width)`` for a layer that appends one
+    ``width``-wide row per token to a paged pool (a latent-attention layer
+    keeps ``[latent | rotated key]``), ``("state", {name: shape})`` for a layer
+    with per-sequence f32 state tensors (``shape`` without the slot axis), or
+    ``None``.  Row pools are ``[num_blocks + 1, block_size, width]`` and state
+    pools ``[num_slots + 1, *shape]``: the last block / slot is a scratch
+    target for padded batch rows.  ``k`` / ``v`` alias the row pools so the
+    engines' device probes (``cache.k[0]``) keep working."""
+
+    def __init__(self, layer_specs, num_blocks: int, num_slots: int, block_size: int = 64,
+                 dtype=torch.bfloat16, device="cuda"):
+        if block_size % 64:
+            raise ValueError("block_size must be a multiple of 64")
+        self.num_layers, self.num_blocks, self.num_slots = len(layer_specs), num_blocks, num_slots
+        self.bs, self.dtype, self.kv_fp8 = block_size, dtype, 0
+        self.k_scale = self.v_scale = 1.0
+        self.device = torch.device(device)
+        self.rows: List[Optional[torch.Tensor]] = []
+        self.state: List[Optional[dict]] = []
+        for spec in layer_specs:
+            rows, st = None, None
+            if spec is not None and spec[0] == "rows":
+                rows = torch.zeros(num_blocks + 1, block_size, int(spec[1]), dtype=dtype, device=device)
+            elif spec is not None and spec[0] == "state":
+                st = {n: torch.zeros(num_slots + 1, *shape, dtype=torch.float32, device=device)
+                      for n, shape in spec[1].items()}
+            self.rows.append(rows)
+            self.state.append(st)
+        probe = next((r for r in self.rows if r is not None), None)
+        if probe is None:
+            probe = torch.zeros(1, dtype=dtype, device=device)
+        self.k = [r if r is not None else probe for r in self.rows]
+        self.v = self.k
+        self.allocator = BlockAllocator(num_blocks)
+        self.slots = SlotAllocator(num_slots)
+
+    def blocks_for(self, n_tokens: int) -> int:
+        return (n_tokens + self.bs - 1) // self.bs
+
+    def bytes(self) -> int:
+        n = sum(r.numel() * r.element_size() for r in self.rows if r is not None)
+        return n + sum(t.numel() * 4 for st in self.state if st for t in st.values())
+
+
 class PagedKVCache:
     def __init__(self, num_layers: int, num_blocks: int, num_kv_heads: int, head_dim: int,
                  block_size: int = 64, dtype=torch.bfloat16, device="cuda", kv_fp8: int = 0,
@@ -61,9 +126,10 @@ class PagedKVCache:
 class SequenceState:
     """Host-side bookkeeping of one sequence in the cache."""
 
-    def __init__(self, blocks: List[int], length: int = 0):
+    def __init__(self, blocks: List[int], length: int = 0, slot: int = -1):
         self.blocks = blocks
         self.length = length
+        self.slot = slot                 # recurrent-state slot (HybridCache), -1: none
 
 
 def make_block_table(seqs: List[SequenceState], max_blocks: int, device) -> torch.Tensor:

@@ -114,6 +114,14 @@ class AttnMeta:
     nsplit: int
     seq_lens_host: Optional[List[int]] = None
     pos_offset: Optional[torch.Tensor] = None   # [B] cache index = pos - offset (compressed KV)
+    # ragged step (models/hybrid.py): sequences bring different numbers of new
+    # tokens (prompt portions beside single decoded tokens); Tq is then the
+    # largest of them and the tokens are laid out sequence after sequence
+    cu_q: Optional[torch.Tensor] = None         # int32 [B + 1] offsets of each sequence's new tokens
+    q_lens_host: Optional[List[int]] = None
+    seq_of: Optional[torch.Tensor] = None       # int32 [T] sequence of every token
+    state_slots: Optional[torch.Tensor] = None  # int32 [B] recurrent-state slot of every sequence
+    prev_ids: Optional[torch.Tensor] = None     # int64 [T] token before each token (-1: none)
 
 
 def interleave_glu_rows(gate: torch.Tensor, up: torch.Tensor, tile: int = 16) -> torch.Tensor:

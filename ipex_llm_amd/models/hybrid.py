@@ -1,0 +1,304 @@
+"""Hybrid decoders: a layer list that mixes attention over a paged cache with
+recurrent layers over per-sequence state, driven by data (``HybridSpec``).
+
+Building blocks (each usable by any design that lists it in its layer specs):
+
+* ``LatentAttention``   low-rank latent attention: one cached row per token,
+  ``[latent c (kv_rank) | shared rotated key (rot_dim)]``; per-head keys and
+  values are ``W_uk c`` / ``W_uv c``, so scores and outputs are formed in the
+  latent space with the up-projections absorbed (as models/mla.py does for
+  the DeepSeek family):  q_lat[h] = W_uk[h]^T q_nope[h],
+  s = (q_lat[h] . c + q_rot[h] . k_rot) scale,  o[h] = W_uv[h] (softmax(s) C).
+  Interleaved-pair rotary positions with optional YaRN scaling, an optional
+  per-head sigmoid output gate.
+* ``MLSTM``             matrix-memory recurrence (xLSTM's mLSTM) with capped
+  exponential gates, running-maximum stabiliser, per-head RMS norm and a
+  sigmoid output gate; f32 state in the cache's slots.
+* ``DenseFF``           gated feed-forward, tanh-GELU.
+
+Block layout (``post_norm`` residual): the sublayers read the residual stream
+``x`` itself and their *output* is normalised:  x += mult * LN(mixer(x)),
+x += mult * LN(ff(x)).  The residual stream is f32 throughout; projections run
+in the model's activation dtype through the vendor GEMM, everything else in
+the kernels of ``ops/seqmix.py``.
+
+``forward_tokens`` takes a *ragged* step (``AttnMeta.cu_q`` ...): sequences
+bring different numbers of new tokens, prompt portions beside single decoded
+tokens, and is what ``serving.engine.LLMEngine`` drives for these models.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Dict, List, Optional
+
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+
+from ..ops import seqmix as SM
+from .decoder import AttnMeta
+
+
+# ---------------------------------------------------------------------- specs
+@dataclass
+class RotarySpec:
+    dims: int
+    base: float = 10000.0
+    scaling: Optional[dict] = None          # YaRN: factor, original, fast, slow
+
+
+@dataclass
+class LatentAttentionSpec:
+    heads: int
+    dim: int                                # unrotated query / key size per head
+    rot_dim: int                            # rotated part (one key shared by all heads)
+    vdim: int
+    kv_rank: int
+    scale: float
+    rot: RotarySpec = None
+    out_gate: bool = True
+
+
+@dataclass
+class MLSTMSpec:
+    heads: int
+    dim: int
+    vdim: int
+    gate_cap: float = 15.0
+
+
+@dataclass
+class DenseFFSpec:
+    ff: int
+
+
+@dataclass
+class LayerSpec:
+    kind: str                               # key of MIXERS
+    mixer: object
+    mlp: Optional[DenseFFSpec] = None
+
+
+@dataclass
+class BigramSpec:
+    buckets: int
+    mul_prev: int
+    mul_cur: int
+
+
+@dataclass
+class HybridSpec:
+    model_type: str
+    vocab_size: int
+    hidden_size: int
+    layers: List[LayerSpec]
+    norm_eps: float = 1e-6
+    residual_mult: float = 1.0
+    bigram: Optional[BigramSpec] = None
+    final_softcap: float = 0.0              # read by the engines' shared helpers
+
+    @property
+    def num_layers(self) -> int:
+        return len(self.layers)
+
+
+# ---------------------------------------------------------------------- mixers
+class LatentAttention(nn.Module):
+    cache_kind = "rows"
+
+    def __init__(self, s: LatentAttentionSpec, w_q, w_dkv, dkv_norm, w_uk, w_uv, w_g, w_o):
+        super().__init__()
+        self.s = s
+        H, r = s.heads, s.kv_rank
+        # one projection launch: [q | dkv | gate] rows
+        parts = [w_q, w_dkv] + ([w_g] if w_g is not None else [])
+        self.w_in = nn.Parameter(torch.cat(parts, 0).contiguous(), requires_grad=False)
+        self.n_q, self.n_dkv = w_q.shape[0], w_dkv.shape[0]
+        self.dkv_norm = nn.Parameter(dkv_norm, requires_grad=False)
+        self.w_uk = nn.Parameter(w_uk.view(H, s.dim, r).contiguous(), requires_grad=False)               # [H, dim, r]
+        self.w_uv_t = nn.Parameter(w_uv.view(H, s.vdim, r).transpose(1, 2).contiguous(), requires_grad=False)  # [H, r, dv]
+        self.w_o = nn.Parameter(w_o, requires_grad=False)
+        self.table: Optional[torch.Tensor] = None
+
+    def cache_spec(self):
+        return ("rows", self.s.kv_rank + self.s.rot_dim)
+
+    def ensure_table(self, max_pos: int):
+        if self.table is None or self.table.shape[0] < max_pos or self.table.device != self.w_o.device:
+            n = max(256, 1 << (max_pos - 1).bit_length())
+            self.table = SM.rope_table(n, self.s.rot.dims, self.s.rot.base, self.s.rot.scaling).to(self.w_o.device)
+        return self.table
+
+    def forward(self, xa, pos, slots, meta: AttnMeta, cache, li: int, eps: float):
+        s = self.s
+        T, H = xa.shape[0], s.heads
+        y = F.linear(xa, self.w_in)
+        q = y[:, :self.n_q].reshape(T, H, s.dim + s.rot_dim).contiguous()
+        dkv = y[:, self.n_q:self.n_q + self.n_dkv]
+        gate = y[:, self.n_q + self.n_dkv:] if s.out_gate else None
+        table = self.table
+        SM.latent_kv_store(dkv, self.dkv_norm, eps, s.kv_rank, table, pos, slots, cache.rows[li])
+        SM.rope_rows_(q, s.dim, table, pos)
+        # absorbed up-projection of the keys: per-head [T, dim] x [dim, r]
+        q_lat = torch.bmm(q[..., :s.dim].transpose(0, 1), self.w_uk).transpose(0, 1)
+        o_lat = SM.latent_attention(q_lat, q[..., s.dim:], cache.rows[li], meta.block_tables, meta.seq_of, pos,
+                                    s.scale, gate, meta.q_lens_host, meta.seq_lens_host, xa.dtype)
+        o = torch.bmm(o_lat.transpose(0, 1), self.w_uv_t).transpose(0, 1).reshape(T, H * s.vdim)
+        return F.linear(o, self.w_o)
+
+
+class MLSTM(nn.Module):
+    cache_kind = "state"
+
+    def __init__(self, s: MLSTMSpec, w_q, w_k, w_v, w_g, w_i, w_f, b_i, b_f, norm, w_o):
+        super().__init__()
+        self.s = s
+        self.w_in = nn.Parameter(torch.cat([w_q, w_k, w_v, w_g, w_i, w_f], 0).contiguous(), requires_grad=False)
+        self.b_i = nn.Parameter(b_i.float(), requires_grad=False)
+        self.b_f = nn.Parameter(b_f.float(), requires_grad=False)
+        self.norm = nn.Parameter(norm, requires_grad=False)
+        self.w_o = nn.Parameter(w_o, requires_grad=False)
+
+    def cache_spec(self):
+        s = self.s
+        return ("state", {"S": (s.heads, s.dim, s.vdim), "n": (s.heads, s.dim), "m": (s.heads,)})
+
+    def ensure_table(self, max_pos: int):
+        return None
+
+    def forward(self, xa, pos, slots, meta: AttnMeta, cache, li: int, eps: float):
+        s = self.s
+        T, H = xa.shape[0], s.heads
+        nqk, nv = H * s.dim, H * s.vdim
+        y = F.linear(xa, self.w_in)
+        q, k = y[:, :nqk].reshape(T, H, s.dim), y[:, nqk:2 * nqk].reshape(T, H, s.dim)
+        v = y[:, 2 * nqk:2 * nqk + nv].reshape(T, H, s.vdim)
+        g = y[:, 2 * nqk + nv:2 * nqk + 2 * nv]
+        ip, fp = y[:, 2 * nqk + 2 * nv:2 * nqk + 2 * nv + H], y[:, 2 * nqk + 2 * nv + H:]
+        h = SM.mlstm_scan(q, k, v, ip, fp, self.b_i, self.b_f, s.gate_cap, cache.state[li], meta.cu_q,
+                          meta.state_slots, pos, meta.q_lens_host)
+        o = SM.head_rms_gate(h, self.norm, g, eps, xa.dtype)
+        return F.linear(o, self.w_o)
+
+
+class DenseFF(nn.Module):
+    def __init__(self, w_gate, w_up, w_down):
+        super().__init__()
+        self.w_gu = nn.Parameter(torch.cat([w_gate, w_up], 0).contiguous(), requires_grad=False)
+        self.w_down = nn.Parameter(w_down, requires_grad=False)
+
+    def forward(self, xa):
+        return F.linear(SM.glu_gelu(F.linear(xa, self.w_gu)), self.w_down)
+
+
+class HybridLayer(nn.Module):
+    def __init__(self, mixer: nn.Module, norm1: torch.Tensor, mlp: Optional[DenseFF], norm2: Optional[torch.Tensor]):
+        super().__init__()
+        self.mixer, self.mlp = mixer, mlp
+        self.norm1 = nn.Parameter(norm1, requires_grad=False)
+        self.norm2 = nn.Parameter(norm2, requires_grad=False) if norm2 is not None else None
+
+
+# name -> (spec class, module class): a design's config reader maps its layer
+# types onto these
+MIXERS: Dict[str, tuple] = {"latent_attention": (LatentAttentionSpec, LatentAttention), "mlstm": (MLSTMSpec, MLSTM)}
+
+
+# ---------------------------------------------------------------------- model
+class HybridCausalLM(nn.Module):
+    ragged_step = True              # forward_tokens takes sequences of unequal new-token counts
+    native_lib = "seqmix"           # the kernels it needs (ops.require_seqmix)
+
+    def __init__(self, spec: HybridSpec, embed: torch.Tensor, bigram: Optional[torch.Tensor],
+                 layers: List[HybridLayer], final_norm: torch.Tensor, head: torch.Tensor, dtype=torch.bfloat16):
+        super().__init__()
+        self.spec, self.dtype = spec, dtype
+        self.embed_tokens = nn.Parameter(embed, requires_grad=False)
+        self.bigram = nn.Parameter(bigram, requires_grad=False) if bigram is not None else None
+        self.layers = nn.ModuleList(layers)
+        self.norm = nn.Parameter(final_norm, requires_grad=False)
+        self.lm_head = nn.Parameter(head, requires_grad=False)
+        self.tp_group = None
+        self.first_stage = self.last_stage = True
+        self.capture_layers: Optional[list] = None      # debugging: residual stream after every layer
+
+    @property
+    def device(self):
+        return self.norm.device
+
+    @property
+    def has_state(self) -> bool:
+        return any(L.mixer.cache_kind == "state" for L in self.layers)
+
+    def graph_max_batch(self) -> int:
+        return 0                    # ragged steps are launched eagerly
+
+    def ensure_rope_cache(self, max_pos: int):
+        for L in self.layers:
+            L.mixer.ensure_table(max_pos)
+
+    def cache_bytes_per_token(self) -> int:
+        eb = torch.empty(0, dtype=self.dtype).element_size()
+        return sum(L.mixer.cache_spec()[1] * eb for L in self.layers if L.mixer.cache_kind == "rows")
+
+    def make_cache(self, max_tokens: int, batch: int = 1, block_size: int = 64, kv_fp8: int = 0,
+                   num_blocks: Optional[int] = None, num_slots: Optional[int] = None):
+        from .cache import HybridCache
+        if kv_fp8:
+            raise ValueError("hybrid decoders keep their latent rows in the activation dtype (no fp8 cache)")
+        nblk = num_blocks or batch * ((max_tokens + block_size - 1) // block_size)
+        self.ensure_rope_cache(max_tokens + 1)
+        return HybridCache([L.mixer.cache_spec() for L in self.layers], nblk, num_slots or batch, block_size,
+                           self.dtype, self.device)
+
+    @staticmethod
+    def complete_meta(meta: AttnMeta, pos: torch.Tensor, T: int) -> AttnMeta:
+        """fill the ragged fields of a uniform (B x Tq) step"""
+        if meta.cu_q is None:
+            dev = pos.device
+            meta.cu_q = torch.arange(0, (meta.B + 1) * meta.Tq, meta.Tq, dtype=torch.int32, device=dev)
+            meta.q_lens_host = [meta.Tq] * meta.B
+            meta.seq_of = torch.arange(meta.B, dtype=torch.int32, device=dev).repeat_interleave(meta.Tq)
+        if meta.seq_lens_host is None:
+            meta.seq_lens_host = [int(v) for v in meta.seq_lens.tolist()]
+        return meta
+
+    def forward_tokens(self, ids: torch.Tensor, pos: torch.Tensor, slots: torch.Tensor, meta: AttnMeta, cache,
+                       logits_idx: Optional[torch.Tensor] = None, return_hidden: bool = False,
+                       hidden_in: Optional[torch.Tensor] = None):
+        """ids / pos / slots [T] (sequence after sequence, ``meta.cu_q``);
+        ``meta.prev_ids`` the token before each one (-1: none) when the model
+        has a bigram table; ``meta.state_slots`` when it has recurrent layers.
+        Returns f32 logits [len(logits_idx) or T, vocab]."""
+        s = self.spec
+        T = ids.shape[0]
+        meta = self.complete_meta(meta, pos, T)
+        if self.has_state and meta.state_slots is None:
+            raise ValueError("a model with recurrent layers needs AttnMeta.state_slots")
+        self.ensure_rope_cache(max(meta.seq_lens_host) + 1)
+        act = self.dtype
+        if hidden_in is not None:
+            x = hidden_in.float().contiguous().clone()
+        elif self.bigram is not None:
+            if meta.prev_ids is None:
+                raise ValueError("a model with a bigram table needs AttnMeta.prev_ids")
+            b = s.bigram
+            x = SM.embed_bigram(ids, meta.prev_ids, self.embed_tokens, self.bigram, b.mul_prev, b.mul_cur)
+        else:
+            x = F.embedding(ids, self.embed_tokens).float()
+        xa = x if act == torch.float32 else x.to(act)
+        for li, L in enumerate(self.layers):
+            y = L.mixer(xa, pos, slots, meta, cache, li, s.norm_eps)
+            xa = SM.add_scaled_layer_norm_(x, y, L.norm1, s.norm_eps, s.residual_mult, act)
+            if L.mlp is not None:
+                xa = SM.add_scaled_layer_norm_(x, L.mlp(xa), L.norm2, s.norm_eps, s.residual_mult, act)
+            if self.capture_layers is not None:
+                self.capture_layers.append(x.clone())
+        if not self.last_stage:
+            return x
+        if logits_idx is not None:
+            x = x.index_select(0, logits_idx)
+        xn = SM.layer_norm_f32(x, self.norm, s.norm_eps, act)
+        if return_hidden:
+            return xn
+        return F.linear(xn, self.lm_head).float()

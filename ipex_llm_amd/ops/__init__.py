@@ -30,6 +30,11 @@ def load(build_if_missing: bool = True) -> bool:
     with _lock:
         if _loaded:
             return True
+        if _seqmix_loaded:
+            # both libraries register the same operators: one per process
+            _load_error = RuntimeError("the sequence-mixing subset library is loaded in this process; "
+                                       "build the full library first (python -m ipex_llm_amd._build) and restart")
+            return False
         try:
             if not os.path.exists(_LIB_PATH) and build_if_missing:
                 from .. import _build
@@ -44,6 +49,38 @@ def load(build_if_missing: bool = True) -> bool:
 
 def available() -> bool:
     return load()
+
+
+# The hybrid decoders (models/hybrid.py) need only the sequence-mixing kernels
+# and the serving scheduler.  Those translation units are part of ``_C.so``
+# and can also be built alone as ``_C_seqmix.so`` (seconds instead of the many
+# minutes of the full library), which is what a checkout without built files
+# compiles when such a model is the first thing it runs.
+_SEQMIX_PATH = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "_C_seqmix.so")
+_seqmix_loaded = False
+
+
+def require_seqmix():
+    """Make ``torch.ops.ipex_llm_amd.sm_*`` and the Scheduler class available:
+    the full library when it is built (or already loaded), else the small
+    sequence-mixing library, built in-tree on first use.  Raises on failure."""
+    global _seqmix_loaded
+    if _loaded or _seqmix_loaded:
+        return torch.ops.ipex_llm_amd
+    with _lock:
+        if _loaded or _seqmix_loaded:
+            return torch.ops.ipex_llm_amd
+        full = os.path.exists(_LIB_PATH)
+    if full:
+        return require()
+    with _lock:
+        from .. import _build
+        stale = _build.needs_build("seqmix")
+        if stale:
+            _build.build(target="seqmix")
+        torch.ops.load_library(_SEQMIX_PATH)
+        _seqmix_loaded = True
+    return torch.ops.ipex_llm_amd
 
 
 def require():

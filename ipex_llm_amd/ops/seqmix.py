@@ -1,0 +1,254 @@
+"""Sequence-mixing ops of the hybrid decoders (models/hybrid.py): latent
+attention over a paged latent cache, the mLSTM matrix-memory recurrence over
+per-sequence state slots, and the element-wise steps around them.
+
+Every op works on a *ragged step*: ``T`` tokens laid out sequence after
+sequence, sequence ``b`` bringing ``cu[b + 1] - cu[b]`` new tokens at
+positions ``pos`` (prompt portions and single decoded tokens side by side).
+GPU tensors run the HIP kernels of ``csrc/hip/seqmix.hip`` (the small
+``_C_seqmix.so`` library, or the full ``_C.so`` which contains them too); CPU
+tensors run the plain torch forms below, which are also what the kernels are
+tested against.
+
+Precision (both paths): positions / angles, attention scores and
+weights, every norm, the residual sum, the recurrence with its gates and its
+state are f32 whatever the activation dtype is; projections and the
+activation of the feed-forward may be 16-bit with f32 accumulation.
+"""
+from __future__ import annotations
+
+import math
+from typing import List, Optional
+
+import torch
+import torch.nn.functional as F
+
+__all__ = ["embed_bigram", "add_scaled_layer_norm_", "layer_norm_f32", "latent_kv_store", "rope_rows_",
+           "latent_attention", "mlstm_scan", "head_rms_gate", "glu_gelu", "rope_table", "native"]
+
+
+def native(t: torch.Tensor) -> bool:
+    """True when ``t`` is a GPU tensor (the HIP kernels must then run)."""
+    if not t.is_cuda:
+        return False
+    from . import require_seqmix
+    require_seqmix()
+    return True
+
+
+def _ops():
+    return torch.ops.ipex_llm_amd
+
+
+# ------------------------------------------------------------------ rotary table
+def rope_table(max_pos: int, dims: int, base: float, scaling: Optional[dict] = None) -> torch.Tensor:
+    """f32 ``[max_pos, dims / 2, 2]`` cos / sin of interleaved-pair rotary
+    positions, angles formed in f64 on the host and rounded once.
+
+    ``scaling`` (YaRN): keys ``factor``, ``original``, ``fast``, ``slow``.
+    With d(t) = dims ln(original / (2 pi t)) / (2 ln base), lo = max(floor(d(fast)), 0),
+    hi = min(ceil(d(slow)), dims - 1) and ramp_i = clamp((i - lo) / max(hi - lo, 1e-3), 0, 1),
+    pair i turns at f_i (1 - ramp_i) + f_i ramp_i / factor, and cos / sin carry
+    the magnitude 0.1 ln(factor) + 1."""
+    i = torch.arange(dims // 2, dtype=torch.float64)
+    f = float(base) ** (-2.0 * i / dims)
+    mag = 1.0
+    if scaling:
+        factor = float(scaling["factor"])
+
+        def d_of(t):
+            return dims * math.log(float(scaling["original"]) / (2 * math.pi * float(t))) / (2 * math.log(float(base)))
+        lo = max(math.floor(d_of(scaling["fast"])), 0)
+        hi = min(math.ceil(d_of(scaling["slow"])), dims - 1)
+        ramp = ((i - lo) / max(hi - lo, 0.001)).clamp(0, 1)
+        f = f / factor * ramp + f * (1 - ramp)
+        mag = 0.1 * math.log(factor) + 1.0
+    a = torch.arange(max_pos, dtype=torch.float64)[:, None] * f[None]
+    return torch.stack([a.cos() * mag, a.sin() * mag], -1).float().contiguous()
+
+
+# ------------------------------------------------------------------ embedding
+def embed_bigram(ids: torch.Tensor, prev_ids: torch.Tensor, embed: torch.Tensor, bigram: torch.Tensor,
+                 mul_prev: int, mul_cur: int) -> torch.Tensor:
+    """f32 ``[T, W]``: ``embed[id] + bigram[row]`` with row = (prev mul_prev +
+    id mul_cur) mod buckets, and the table's last row (index ``buckets``) for a
+    token without a predecessor (``prev_ids < 0``)."""
+    buckets = bigram.shape[0] - 1
+    if native(ids):
+        return _ops().sm_embed_bigram(ids.contiguous(), prev_ids.contiguous(), embed, bigram, mul_prev, mul_cur)
+    row = (prev_ids.long() * mul_prev + ids.long() * mul_cur) % buckets
+    row = torch.where(prev_ids < 0, torch.full_like(row, buckets), row)
+    return embed[ids].float() + bigram[row].float()
+
+
+# ------------------------------------------------------------------ norms
+def add_scaled_layer_norm_(x: torch.Tensor, y: torch.Tensor, w: torch.Tensor, eps: float, mult: float,
+                           act_dtype: torch.dtype) -> torch.Tensor:
+    """``x += mult * LN(y) * w`` on the f32 residual stream ``x`` in place
+    (LN without bias, variance = mean squared deviation); returns ``x`` in
+    ``act_dtype`` for the next projection (``x`` itself when that is f32)."""
+    if native(x):
+        return _ops().sm_add_scaled_layer_norm(x, y.contiguous(), w, eps, mult, act_dtype == torch.float32)
+    yf = y.float()
+    mu = yf.mean(-1, keepdim=True)
+    d = yf - mu
+    x.add_(d * torch.rsqrt((d * d).mean(-1, keepdim=True) + eps) * w.float() * mult)
+    return x if act_dtype == torch.float32 else x.to(act_dtype)
+
+
+def layer_norm_f32(x: torch.Tensor, w: torch.Tensor, eps: float, act_dtype: torch.dtype) -> torch.Tensor:
+    """bias-free LayerNorm of f32 rows, result in ``act_dtype``."""
+    if native(x):
+        return _ops().sm_layer_norm(x.contiguous(), w, eps, act_dtype == torch.float32)
+    mu = x.mean(-1, keepdim=True)
+    d = x - mu
+    return (d * torch.rsqrt((d * d).mean(-1, keepdim=True) + eps) * w.float()).to(act_dtype)
+
+
+# ------------------------------------------------------------------ rotary
+def _rot_pairs(x: torch.Tensor, cs: torch.Tensor) -> torch.Tensor:
+    """x f32 [..., dims] interleaved pairs, cs [..., dims / 2, 2]"""
+    u, v = x[..., 0::2], x[..., 1::2]
+    c, s = cs[..., 0], cs[..., 1]
+    return torch.stack([u * c - v * s, v * c + u * s], -1).flatten(-2)
+
+
+def rope_rows_(q: torch.Tensor, offset: int, table: torch.Tensor, pos: torch.Tensor) -> torch.Tensor:
+    """Rotate, in place, the ``dims = 2 * table.shape[1]`` values of every head
+    of ``q`` [T, H, D] that start at ``offset`` (interleaved pairs, f32 math)."""
+    dims = 2 * table.shape[1]
+    if native(q):
+        _ops().sm_rope_rows_(q, offset, table, pos)
+        return q
+    cs = table[pos.long()][:, None]                                 # [T, 1, dims / 2, 2]
+    q[..., offset:offset + dims] = _rot_pairs(q[..., offset:offset + dims].float(), cs).to(q.dtype)
+    return q
+
+
+def latent_kv_store(dkv: torch.Tensor, norm_w: torch.Tensor, eps: float, rank: int, table: torch.Tensor,
+                    pos: torch.Tensor, slots: torch.Tensor, rows: torch.Tensor) -> None:
+    """One cache row per token: ``[rms_norm(dkv[:rank]) * norm_w | rope(dkv[rank:])]``
+    written at row index ``slots`` of the paged pool ``rows`` [blocks, bs, width]
+    (the rotation covers the first ``2 * table.shape[1]`` values of the rotated part)."""
+    if native(dkv):
+        _ops().sm_latent_kv_store(dkv, norm_w, eps, rank, table, pos, slots, rows)
+        return
+    dims = 2 * table.shape[1]
+    c = dkv[:, :rank].float()
+    c = c * torch.rsqrt((c * c).mean(-1, keepdim=True) + eps) * norm_w.float()
+    kr = dkv[:, rank:].float().clone()
+    kr[:, :dims] = _rot_pairs(kr[:, :dims], table[pos.long()])
+    flat = rows.view(-1, rows.shape[-1])
+    flat.index_copy_(0, slots.long(), torch.cat([c, kr], -1).to(rows.dtype))
+
+
+# ------------------------------------------------------------------ latent attention
+def latent_attention(q_lat: torch.Tensor, q_rot: torch.Tensor, rows: torch.Tensor, block_tables: torch.Tensor,
+                     seq_of: torch.Tensor, pos: torch.Tensor, scale: float, gate: Optional[torch.Tensor],
+                     q_lens: List[int], ctx_lens: List[int], out_dtype: torch.dtype) -> torch.Tensor:
+    """Causal softmax attention in the latent space over the paged rows
+    ``[latent (r) | rotated key (dr)]``: for token t of sequence b and head h
+
+        s_j = (q_lat[t, h] . c_j + q_rot[t, h] . kr_j) * scale      for j <= pos[t]
+        out[t, h] = sigmoid(gate[t, h]) * sum_j softmax(s)_j c_j     [r]
+
+    (scores, softmax and the weighted sum in f32).  ``q_rot`` may be a strided
+    view.  ``q_lens`` / ``ctx_lens``: host copies of every sequence's new-token
+    count and key count."""
+    T, H, r = q_lat.shape
+    if native(q_lat):
+        return _ops().sm_latent_attention(q_lat.contiguous(), q_rot, rows, block_tables, seq_of, pos, float(scale),
+                                          gate, max(ctx_lens), out_dtype == torch.float32)
+    out = torch.empty(T, H, r, dtype=torch.float32, device=q_lat.device)
+    bs = rows.shape[1]
+    t0 = 0
+    for b, (n, L) in enumerate(zip(q_lens, ctx_lens)):
+        if n == 0:
+            continue
+        nb = (L + bs - 1) // bs
+        kv = rows[block_tables[b, :nb].long()].reshape(nb * bs, -1)[:L].float()
+        c, kr = kv[:, :r], kv[:, r:]
+        ql, qr = q_lat[t0:t0 + n].float(), q_rot[t0:t0 + n].float()
+        sc = (torch.einsum("thr,lr->thl", ql, c) + torch.einsum("thd,ld->thl", qr, kr)) * scale
+        vis = torch.arange(L, device=sc.device)[None, :] <= pos[t0:t0 + n].long()[:, None]
+        sc = sc.masked_fill(~vis[:, None, :], float("-inf"))
+        out[t0:t0 + n] = torch.einsum("thl,lr->thr", torch.softmax(sc, -1), c)
+        t0 += n
+    if gate is not None:
+        out = out * torch.sigmoid(gate.float())[..., None]
+    return out.to(out_dtype)
+
+
+# ------------------------------------------------------------------ mLSTM
+def mlstm_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, i_pre: torch.Tensor, f_pre: torch.Tensor,
+               i_bias: torch.Tensor, f_bias: torch.Tensor, cap: float, state: dict, cu: torch.Tensor,
+               state_slots: torch.Tensor, pos: torch.Tensor, q_lens: List[int]) -> torch.Tensor:
+    """Matrix-memory recurrence, token by token, per sequence and head.
+
+    q, k [T, H, d], v [T, H, dv], gate pre-activations [T, H]; ``state`` holds
+    f32 ``S`` [slots, H, d, dv], ``n`` [slots, H, d], ``m`` [slots, H], read at
+    ``state_slots[b]`` (a sequence whose first new token is at position 0
+    starts from zero instead) and written back after the last token.  With
+    i = cap tanh((i_pre + b_i) / cap), f = logsigmoid(cap tanh((f_pre + b_f) / cap)):
+
+        m' = max(f + m, i);  a = exp(f + m - m');  b = exp(i - m')
+        S' = a S + b k v^T;  n' = a n + b k
+        h  = S'^T q' / (max(|n' . q'|, exp(-m')) + 1e-6),   q' = q d^-1/2
+
+    Returns h f32 [T, H, dv]."""
+    T, H, d = q.shape
+    dv = v.shape[-1]
+    if native(q):
+        return _ops().sm_mlstm_scan(q, k, v, i_pre, f_pre, i_bias, f_bias, float(cap), state["S"], state["n"],
+                                    state["m"], cu, state_slots, pos, max(q_lens))
+    out = torch.empty(T, H, dv, dtype=torch.float32, device=q.device)
+    ig = cap * torch.tanh((i_pre.float() + i_bias.float()) / cap)
+    fg = F.logsigmoid(cap * torch.tanh((f_pre.float() + f_bias.float()) / cap))
+    qf, kf, vf = q.float() * d ** -0.5, k.float(), v.float()
+    slots = state_slots.tolist()
+    first = pos.tolist()
+    t0 = 0
+    for b, nq in enumerate(q_lens):
+        if nq == 0:
+            continue
+        sl = slots[b]
+        if first[t0] == 0:
+            S = torch.zeros(H, d, dv, device=q.device)
+            n = torch.zeros(H, d, device=q.device)
+            m = torch.zeros(H, device=q.device)
+        else:
+            S, n, m = state["S"][sl].clone(), state["n"][sl].clone(), state["m"][sl].clone()
+        for t in range(t0, t0 + nq):
+            mn = torch.maximum(fg[t] + m, ig[t])
+            a, bb = torch.exp(fg[t] + m - mn), torch.exp(ig[t] - mn)
+            S = a[:, None, None] * S + bb[:, None, None] * kf[t][:, :, None] * vf[t][:, None, :]
+            n = a[:, None] * n + bb[:, None] * kf[t]
+            m = mn
+            den = torch.maximum((n * qf[t]).sum(-1).abs(), torch.exp(-m)) + 1e-6
+            out[t] = torch.einsum("hdv,hd->hv", S, qf[t]) / den[:, None]
+        state["S"][sl], state["n"][sl], state["m"][sl] = S, n, m
+        t0 += nq
+    return out
+
+
+def head_rms_gate(h: torch.Tensor, norm_w: torch.Tensor, gate_pre: torch.Tensor, eps: float,
+                  out_dtype: torch.dtype) -> torch.Tensor:
+    """h f32 [T, H, dv]: every head divided by its root mean square, then
+    ``* norm_w`` (all heads' size) ``* sigmoid(gate_pre)`` -> [T, H * dv]."""
+    T, H, dv = h.shape
+    if native(h):
+        return _ops().sm_head_rms_gate(h.contiguous(), norm_w, gate_pre, eps, out_dtype == torch.float32)
+    y = h * torch.rsqrt((h * h).mean(-1, keepdim=True) + eps)
+    y = y.reshape(T, H * dv) * norm_w.float() * torch.sigmoid(gate_pre.float())
+    return y.to(out_dtype)
+
+
+# ------------------------------------------------------------------ feed-forward
+def glu_gelu(gu: torch.Tensor) -> torch.Tensor:
+    """[T, 2 I] = [gate | up] -> gelu_tanh(gate) * up  [T, I] (f32 math)."""
+    I = gu.shape[-1] // 2
+    if native(gu):
+        return _ops().sm_glu_gelu(gu.contiguous())
+    g, u = gu[..., :I].float(), gu[..., I:].float()
+    a = 0.5 * g * (1.0 + torch.tanh(math.sqrt(2.0 / math.pi) * (g + 0.044715 * g * g * g)))
+    return (a * u).to(gu.dtype)

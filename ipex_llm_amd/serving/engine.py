@@ -62,7 +62,14 @@ class LLMEngine:
                  num_blocks: Optional[int] = None, max_model_len: int = 8192, max_prefill_tokens: int = 8192,
                  kv_fp8: int = 0, memory_fraction: float = 0.5, eos_token_id=None, use_graph: bool = True,
                  enable_prefix_caching: bool = True, tp_group="auto"):
-        ops.require() if model.device.type == "cuda" else None
+        # models whose forward takes ragged steps (prompt portions beside
+        # decoded tokens in one batch, models/hybrid.py) run mixed, chunked
+        # steps; they name the kernel library they need
+        self.ragged = bool(getattr(model, "ragged_step", False))
+        if model.device.type == "cuda":
+            ops.require_seqmix() if getattr(model, "native_lib", None) == "seqmix" else ops.require()
+        elif self.ragged:
+            ops.require_seqmix()               # the scheduler class lives in the native library
         self.model = model
         s = model.spec
         # tensor-parallel serving (reference: vLLM --tensor-parallel-size,
@@ -83,7 +90,8 @@ class LLMEngine:
         self.is_driver = self.tp_rank == 0
         self._stopped = False
         if num_blocks is None:
-            per_tok = PagedKVCache.bytes_per_token(len(model.layers), s.num_kv_heads, s.head_dim, model.dtype, kv_fp8)
+            per_tok = max(1, model.cache_bytes_per_token()) if hasattr(model, "cache_bytes_per_token") else \
+                PagedKVCache.bytes_per_token(len(model.layers), s.num_kv_heads, s.head_dim, model.dtype, kv_fp8)
             if model.device.type == "cuda":
                 free, _ = torch.cuda.mem_get_info(model.device)
                 budget = int(free * memory_fraction)
@@ -95,19 +103,25 @@ class LLMEngine:
                 num_blocks = int(self._tp_reduce_min(num_blocks))
         # one extra block past the scheduler's pool: the scratch target of the
         # padding rows of a captured decode step
-        self.cache = model.make_cache(max_model_len, max_batch, block_size, kv_fp8, num_blocks=num_blocks + 1)
+        if self.ragged:
+            # the pool as asked (the cache adds its own scratch block / slot)
+            self.cache = model.make_cache(max_model_len, max_batch, block_size, kv_fp8, num_blocks=num_blocks,
+                                          num_slots=max_batch)
+        else:
+            self.cache = model.make_cache(max_model_len, max_batch, block_size, kv_fp8, num_blocks=num_blocks + 1)
         self._scratch = num_blocks
         self.num_blocks = num_blocks
         # prefill GEMMs on a resident dequantized shadow (ops/gemm.py
         # auto_dense_budget), bounded by half of what the KV pool left free
         self.prefill_dense_gb = 0.0
-        if model.device.type == "cuda":
+        if model.device.type == "cuda" and not self.ragged:
             from ..ops.gemm import auto_dense_budget
             free, _ = torch.cuda.mem_get_info(model.device)
             self.prefill_dense_gb = auto_dense_budget(model.device, cap_gb=0.5 * free / 2 ** 30)
         from .metrics import EngineMetrics
         self.metrics = EngineMetrics()
-        self.use_graph = use_graph and model.device.type == "cuda" and ops.native_gpu(self.cache.k[0])
+        self.use_graph = use_graph and not self.ragged and model.device.type == "cuda" and \
+            ops.native_gpu(self.cache.k[0])
         self._graphs: Dict[tuple, dict] = {}
         # every captured (batch, width) bucket allocates from ONE private pool,
         # and only buckets whose forward is capture-safe are captured (MoE
@@ -118,8 +132,14 @@ class LLMEngine:
         self.sched = torch.classes.ipex_llm_amd.Scheduler(num_blocks, block_size, max_batch, max_prefill_tokens)
         # automatic prefix caching: full KV blocks are shared by content hash
         # (C++ scheduler); a request prefills only its uncached suffix
-        self.prefix_caching = bool(enable_prefix_caching)
+        # (mixed steps admit without prefix matching, and recurrent state could
+        # not be rebuilt from shared KV blocks anyway: no prefix reuse there)
+        self.prefix_caching = bool(enable_prefix_caching) and not self.ragged
         self.sched.enable_prefix_caching(self.prefix_caching)
+        if self.ragged:
+            self.sched.set_state_slots(max_batch)
+        self._streams: Dict[int, int] = {}      # externally fed sequences (open_stream)
+        self._last_tok: Dict[int, int] = {}     # last token run of every sequence (bigram embeddings)
         self.block_size, self.max_model_len = block_size, max_model_len
         eos = eos_token_id if eos_token_id is not None else []
         self.eos = set([eos] if isinstance(eos, int) else eos)
@@ -163,6 +183,7 @@ class LLMEngine:
     # ------------------------------------------------------------ step
     def _finish(self, r: Request, reason: str):
         r.finished, r.finish_reason = True, reason
+        self._last_tok.pop(r.rid, None)
         self.metrics.on_finish(reason, time.perf_counter() - r.arrival, len(r.generated), r.first_token_time)
         try:
             self.sched.finish(r.rid)
@@ -363,6 +384,126 @@ class LLMEngine:
         meta = AttnMeta(B, 1, bt, seq_lens, nsplit_for(max(pos_l) + 1), [p + 1 for p in pos_l])
         return m.forward_tokens(torch.tensor(ids_l, device=dev), pos, slots, meta, self.cache)
 
+    # ------------------------------------------------------------ ragged steps
+    @torch.no_grad()
+    def run_batch(self, entries) -> torch.Tensor:
+        """One forward over a mixed batch: ``entries`` is a list of
+        ``(rid, tokens, want)`` -- the next tokens of running sequence ``rid``
+        (a portion of its prompt, or one decoded token) and the indices among
+        them whose logits are wanted.  Every sequence continues from what the
+        cache and its state slot hold (``sched.cached(rid)`` tokens); all
+        entries run together.  Returns f32 logits [sum(len(want)), vocab] in
+        entry order and marks the tokens as cached."""
+        if not self.ragged:
+            raise RuntimeError("run_batch: this model's forward takes uniform batches only")
+        m, dev, bs = self.model, self.model.device, self.block_size
+        ids, pos, slots, seq_of, prev, lidx = [], [], [], [], [], []
+        cu, ctx, qn, rows, sslots = [0], [], [], [], []
+        for b, (rid, toks, want) in enumerate(entries):
+            n = len(toks)
+            if n == 0:
+                raise ValueError("run_batch: an entry without tokens")
+            start = int(self.sched.cached(rid))
+            blocks = list(self.sched.blocks(rid))
+            if start + n > len(blocks) * bs:
+                raise RuntimeError(f"run_batch: sequence {rid} has no blocks for {start + n} tokens")
+            last = self._last_tok.get(rid, -1) if start > 0 else -1
+            for i, t in enumerate(toks):
+                p = start + i
+                ids.append(int(t))
+                pos.append(p)
+                slots.append(blocks[p // bs] * bs + p % bs)
+                prev.append(last)
+                last = int(t)
+            seq_of += [b] * n
+            lidx += [cu[-1] + int(w) for w in want]
+            cu.append(cu[-1] + n)
+            ctx.append(start + n)
+            qn.append(n)
+            rows.append(blocks)
+            sslots.append(max(int(self.sched.slot(rid)), 0))
+        w = max(len(x) for x in rows)
+        bt = torch.full((len(rows), w), self._scratch, dtype=torch.int32)
+        for i, x in enumerate(rows):
+            bt[i, :len(x)] = torch.tensor(x, dtype=torch.int32)
+        i32 = lambda v: torch.tensor(v, dtype=torch.int32, device=dev)      # noqa: E731
+        i64 = lambda v: torch.tensor(v, dtype=torch.long, device=dev)       # noqa: E731
+        meta = AttnMeta(len(entries), max(qn), bt.to(dev), i32(ctx), nsplit_for(max(ctx)), list(ctx),
+                        cu_q=i32(cu), q_lens_host=qn, seq_of=i32(seq_of), state_slots=i32(sslots), prev_ids=i64(prev))
+        logits = m.forward_tokens(i64(ids), i64(pos), i64(slots), meta, self.cache, logits_idx=i64(lidx))
+        for rid, toks, _ in entries:
+            self.sched.advance(rid, len(toks))
+            self._last_tok[rid] = int(toks[-1])
+        return logits
+
+    def open_stream(self) -> int:
+        """Admit a sequence whose tokens are fed from outside with
+        ``run_batch`` (its length is not known up front: blocks are taken as
+        it grows).  Returns its id; ``close_stream`` gives everything back."""
+        with self.lock:
+            rid = next(self._ids)
+            self.sched.open(rid)
+            self._streams[rid] = -1
+            return rid
+
+    def feed(self, entries) -> torch.Tensor:
+        """``run_batch`` for streams: takes the blocks the new tokens need first."""
+        with self.lock:
+            for rid, toks, _ in entries:
+                self.sched.extend(rid, len(toks))
+            return self.run_batch(entries)
+
+    def close_stream(self, rid: int):
+        with self.lock:
+            self._streams.pop(rid, None)
+            self._last_tok.pop(rid, None)
+            self.sched.finish(rid)
+
+    def _step_ragged(self) -> int:
+        """Scheduler step of a ragged model: one mixed forward -- every running
+        sequence brings its next token or the next portion of its prompt
+        (``max_prefill_tokens`` per step in all)."""
+        t_step = time.perf_counter()
+        with self.lock:
+            plan = list(self.sched.schedule_mixed())
+            i1 = plan.index(-1)
+            i2 = plan.index(-1, i1 + 1)
+            work, preempted, failed = plan[:i1], plan[i1 + 1:i2], plan[i2 + 1:]
+            self.stats["preemptions"] += len(preempted)
+            for rid in failed:
+                r = self.requests[rid]
+                r.finished, r.finish_reason = True, "error: request does not fit in the KV cache"
+                if r.on_token is not None:
+                    r.on_token(-1, r)
+            entries, done = [], []
+            for rid, n in zip(work[0::2], work[1::2]):
+                r = self.requests[rid]
+                start = int(self.sched.cached(rid))
+                last = start + n == len(r.tokens)
+                entries.append((rid, r.tokens[start:start + n], [n - 1] if last else []))
+                done.append(last)
+                npre = min(start + n, len(r.prompt)) - start
+                if npre > 0:
+                    self.stats["prefill_tokens"] += npre
+                    self.metrics.on_prefill(npre)
+            produced = 0
+            if entries:
+                lg = self.run_batch(entries)
+                rs = [self.requests[e[0]] for e, d in zip(entries, done) if d]
+                if rs:
+                    greedy = all(not r.params.do_sample and r.params.repetition_penalty == 1.0 for r in rs)
+                    nxt = torch.argmax(lg, -1).tolist() if greedy else None
+                    for i, r in enumerate(rs):
+                        self._emit(r, nxt[i] if greedy else self._pick(lg[i:i + 1], r))
+                    produced = len(rs)
+                    self.stats["decode_tokens"] += produced
+            self.stats["steps"] += 1
+            self.metrics.on_tokens(produced)
+            self.metrics.on_step(time.perf_counter() - t_step, int(self.sched.num_running()),
+                                 int(self.sched.num_waiting()),
+                                 1.0 - int(self.sched.num_free_blocks()) / max(1, self.num_blocks), len(preempted))
+            return produced
+
     @torch.no_grad()
     def step(self) -> int:
         """One scheduler step: prefill admitted requests, decode all running
@@ -374,6 +515,8 @@ class LLMEngine:
     def _step(self) -> int:
         if not self.is_driver:
             raise RuntimeError("LLMEngine.step: tensor-parallel ranks > 0 run run_worker(), not step()")
+        if self.ragged:
+            return self._step_ragged()
         t_step = time.perf_counter()
         with self.lock:
             plan = list(self.sched.schedule())
