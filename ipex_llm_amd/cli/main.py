@@ -17,6 +17,11 @@ import time
 def _load(args):
     import torch
     from ..transformers import AutoModelForCausalLM
+    from ..models.registry import NativeCheckpointLM, native_architecture
+    if native_architecture(args.model) is not None:
+        # native checkpoint layouts carry no tokenizer: prompts are token ids (--prompt-ids)
+        return NativeCheckpointLM(args.model, torch.bfloat16 if args.device != "cpu" else torch.float32,
+                                  args.device), None
     if getattr(args, "load_low_bit", False):
         model = AutoModelForCausalLM.load_low_bit(args.model)
     elif args.model.endswith(".gguf"):
@@ -32,6 +37,17 @@ def _load(args):
 
 def cmd_generate(args):
     model, tok = _load(args)
+    if tok is None or args.prompt_ids:
+        if not args.prompt_ids:
+            raise SystemExit("generate: this checkpoint has no tokenizer; give --prompt-ids 1,2,3")
+        rows = [[int(t) for t in args.prompt_ids.replace(" ", "").split(",") if t]]
+        t0 = time.perf_counter()
+        out = model.generate(rows, max_new_tokens=args.n_predict, do_sample=args.temperature > 0,
+                             temperature=max(args.temperature, 1e-5))
+        out = out.tolist() if hasattr(out, "tolist") else out
+        print(",".join(str(t) for t in out[0][len(rows[0]):]))
+        print(f"\n[{len(out[0]) - len(rows[0])} tokens, {time.perf_counter() - t0:.2f} s]", file=sys.stderr)
+        return
     ids = tok(args.prompt, return_tensors="pt").input_ids.to(args.device)
     t0 = time.perf_counter()
     out = model.generate(ids, max_new_tokens=args.n_predict, do_sample=args.temperature > 0,
@@ -99,7 +115,10 @@ def main(argv=None):
 
     g = sub.add_parser("generate", help="one completion (llm-cli)")
     model_args(g)
-    g.add_argument("-p", "--prompt", required=True)
+    g.add_argument("-p", "--prompt", default=None)
+    g.add_argument("--prompt-ids", default=None, help="comma-separated token ids instead of text")
+    tr = sub.add_parser("trace", help="replay token steps from stdin and write logits (bin/trace_run)")
+    tr.add_argument("rest", nargs=argparse.REMAINDER)
     c = sub.add_parser("chat", help="interactive chat (llm-chat)")
     model_args(c)
     s = sub.add_parser("serve", help="OpenAI-compatible HTTP server")
@@ -145,7 +164,12 @@ def main(argv=None):
         r = strided_perplexity(model, text_ids(tok, a.data_path, a.max_tokens), a.chunk_size, a.stride or None)
         print(json.dumps({"model": a.model_path, "precision": a.precision, **r}))
         return r
+    if a.cmd == "trace":
+        from .trace import main as trace_main
+        return trace_main(a.rest)
     if a.cmd == "generate":
+        if a.prompt is None and not a.prompt_ids:
+            ap.error("generate: give --prompt or --prompt-ids")
         return cmd_generate(a)
     if a.cmd == "chat":
         return cmd_chat(a)

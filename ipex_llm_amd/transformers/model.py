@@ -177,6 +177,13 @@ class _BaseAutoModelClass:
     def from_pretrained(cls, *args, **kwargs):
         path = kwargs.pop("pretrained_model_name_or_path", None) if not args else args[0]
         args = args[1:] if args else ()
+        from ..models.registry import NativeCheckpointLM, native_architecture
+        if path is not None and native_architecture(path) is not None:
+            # a checkpoint in a native layout (models/registry.py): no HF class,
+            # no conversion -- loaded as stored and served by the engine
+            dt = kwargs.get("torch_dtype", kwargs.get("dtype", None))
+            dt = dt if isinstance(dt, torch.dtype) else torch.bfloat16
+            return NativeCheckpointLM(path, dtype=dt, device=kwargs.get("device", "cpu"))
         qtype = _resolve_qtype_from_kwargs(kwargs)
         optimize_model = kwargs.pop("optimize_model", True)
         modules_to_not_convert = kwargs.pop("modules_to_not_convert", None)
