@@ -158,7 +158,17 @@ def main():
     ap.add_argument("--ep", action="store_true", help="expert parallel over all ranks (MoE models)")
     ap.add_argument("--no-tp-side", action="store_true",
                     help="N > 1 data-parallel run: skip the tensor-parallel (strong-scaling) side measurement")
+    ap.add_argument("--hybrid", action="store_true",
+                    help="side benchmark (not the headline metric): prefill / decode throughput of the hybrid "
+                         "latent-attention + mLSTM decoder beside the MLA decoder at equal sizes, one GPU")
+    ap.add_argument("--hybrid-sizes", default="small,base")
+    ap.add_argument("--hybrid-prompts", default="1024,4096")
+    ap.add_argument("--no-hybrid-ref", action="store_true", help="--hybrid: skip the MLA comparison model")
     args = ap.parse_args()
+    if args.hybrid:
+        from ipex_llm_amd.utils.bench_hybrid import main as hybrid_main
+        hybrid_main(args)
+        return
 
     world = int(os.environ.get("WORLD_SIZE", "1"))
     rank = int(os.environ.get("RANK", "0"))

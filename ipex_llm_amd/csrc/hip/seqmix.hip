@@ -170,34 +170,56 @@ __global__ void __launch_bounds__(128) latent_kv_store_k(const E* __restrict__ d
 // token's key tiles (KT keys each, tile i -> keys [i KT, (i + 1) KT), always
 // inside one cache page) round-robin; a wave stages a tile in LDS, lane j
 // scores key j against every head (f32), the wave does the online-softmax
-// update per head, and every lane accumulates its latent columns.  The waves'
+// update per head, and every lane accumulates its latent columns (f32
+// weights x latents: the weights are never rounded to 16 bits).  The waves'
 // partial (max, sum, out) are merged through LDS at the end.
-constexpr int HB = 8;
+// LDS rows are padded to DP = 4 (mod 8) elements: 4-element reads of one
+// column group by 64 lanes then spread over all banks.
+template <typename E> struct Ld4;
+template <> struct Ld4<float> {
+  static __device__ __forceinline__ void get(const float* p, float* o) {
+    const float4 v = *(const float4*)p;
+    o[0] = v.x; o[1] = v.y; o[2] = v.z; o[3] = v.w;
+  }
+};
+template <> struct Ld4<__bf16> {
+  static __device__ __forceinline__ void get(const __bf16* p, float* o) {
+    const uint2 v = *(const uint2*)p;
+    o[0] = __uint_as_float(v.x << 16); o[1] = __uint_as_float(v.x & 0xffff0000u);
+    o[2] = __uint_as_float(v.y << 16); o[3] = __uint_as_float(v.y & 0xffff0000u);
+  }
+};
 
-template <typename E, int RC>
+template <typename E, int RC, int HB>
 __global__ void __launch_bounds__(256) latent_attn_k(const E* __restrict__ q_lat, const E* __restrict__ q_rot,
                                                     int64_t qr_st, int64_t qr_sh, const E* __restrict__ rows, int bs,
                                                     const int32_t* __restrict__ bt, int bt_w,
                                                     const int32_t* __restrict__ seq_of, const int64_t* __restrict__ pos,
                                                     float scale, const E* __restrict__ gate, int64_t g_st,
-                                                    E* __restrict__ out, int H, int r, int dr, int KT, int DP) {
+                                                    E* __restrict__ out, float* __restrict__ part, int H, int r, int dr,
+                                                    int KT, int DP) {
   extern __shared__ __align__(16) unsigned char smem[];
-  const int D = r + dr;
+  const int D = r + dr, D4 = (D + 3) & ~3;
+  const int nsplit = gridDim.z, zs = blockIdx.z;
   const int t = blockIdx.x, h0 = blockIdx.y * HB;
   const int nh = min(HB, H - h0);
   const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6, NW = blockDim.x >> 6;
-  float* qs = (float*)smem;                                        // [HB][D]
+  E* qs = (E*)smem;                                                // [HB][D4], zero padded
+  const size_t q_bytes = ((size_t)HB * D4 * sizeof(E) + 15) & ~(size_t)15;
   const size_t wave_bytes = ((size_t)KT * DP * sizeof(E) + (size_t)HB * KT * sizeof(float) + 15) & ~(size_t)15;
-  unsigned char* wbase = smem + (((size_t)HB * D * sizeof(float) + 15) & ~(size_t)15) + wv * wave_bytes;
+  unsigned char* wbase = smem + q_bytes + wv * wave_bytes;
   E* kt = (E*)wbase;                                               // [KT][DP]
   float* pb = (float*)(wbase + (size_t)KT * DP * sizeof(E));       // [HB][KT]
-  for (int i = threadIdx.x; i < HB * D; i += blockDim.x) {
-    const int h = i / D, c = i - h * D;
+  for (int i = threadIdx.x; i < HB * D4; i += blockDim.x) {
+    const int h = i / D4, c = i - h * D4;
     float v = 0.f;
-    if (h < nh) v = c < r ? ldf(q_lat + ((int64_t)t * H + h0 + h) * r + c)
-                          : ldf(q_rot + (int64_t)t * qr_st + (int64_t)(h0 + h) * qr_sh + (c - r));
-    qs[i] = v;
+    if (h < nh && c < D)
+      v = c < r ? ldf(q_lat + ((int64_t)t * H + h0 + h) * r + c)
+                : ldf(q_rot + (int64_t)t * qr_st + (int64_t)(h0 + h) * qr_sh + (c - r));
+    stf(qs + i, v);
   }
+  // the whole tile buffer starts finite: rows and pad columns a tile does not fill are read with weight 0
+  for (int i = lane; i < KT * DP; i += 64) stf(kt + i, 0.f);
   __syncthreads();
   const int64_t p = pos[t];
   const int32_t* tab = bt + (int64_t)seq_of[t] * bt_w;
@@ -210,7 +232,7 @@ __global__ void __launch_bounds__(256) latent_attn_k(const E* __restrict__ q_lat
 #pragma unroll
     for (int c = 0; c < RC; c++) o[h][c] = 0.f;
   }
-  for (int ti = wv; ti < ntiles; ti += NW) {
+  for (int ti = zs * NW + wv; ti < ntiles; ti += NW * nsplit) {
     const int64_t k0 = (int64_t)ti * KT;
     const int nvalid = (int)min((int64_t)KT, p - k0 + 1);
     const int64_t row0 = (int64_t)tab[k0 / bs] * bs + (k0 % bs);
@@ -226,10 +248,15 @@ __global__ void __launch_bounds__(256) latent_attn_k(const E* __restrict__ q_lat
     const bool valid = lane < nvalid;
     if (valid) {
       const E* kr = kt + lane * DP;
-      for (int c = 0; c < D; c++) {
-        const float kv = ldf(kr + c);
+      for (int c = 0; c < D4; c += 4) {
+        float kv[4];
+        Ld4<E>::get(kr + c, kv);
 #pragma unroll
-        for (int h = 0; h < HB; h++) s[h] = fmaf(qs[h * D + c], kv, s[h]);
+        for (int h = 0; h < HB; h++) {
+          float qv[4];
+          Ld4<E>::get(qs + h * D4 + c, qv);
+          s[h] = fmaf(qv[0], kv[0], fmaf(qv[1], kv[1], fmaf(qv[2], kv[2], fmaf(qv[3], kv[3], s[h]))));
+        }
       }
     }
 #pragma unroll
@@ -245,24 +272,31 @@ __global__ void __launch_bounds__(256) latent_attn_k(const E* __restrict__ q_lat
       if (lane < KT) pb[h * KT + lane] = pv;
     }
     wave_sync();
-    for (int j = 0; j < nvalid; j++) {
-      float kv[RC];
+    const int nv4 = (nvalid + 3) & ~3;                             // weights past nvalid are 0, rows finite
+    for (int j = 0; j < nv4; j += 4) {
+      float kv[4][RC];
 #pragma unroll
-      for (int c = 0; c < RC; c++) {
-        const int col = lane + 64 * c;
-        kv[c] = col < r ? ldf(kt + j * DP + col) : 0.f;
-      }
+      for (int jj = 0; jj < 4; jj++)
+#pragma unroll
+        for (int c = 0; c < RC; c++) {
+          const int col = lane + 64 * c;
+          kv[jj][c] = col < r ? ldf(kt + (j + jj) * DP + col) : 0.f;
+        }
 #pragma unroll
       for (int h = 0; h < HB; h++) {
-        const float pv = pb[h * KT + j];
+        const float4 pv = *(const float4*)(pb + h * KT + j);
 #pragma unroll
-        for (int c = 0; c < RC; c++) o[h][c] = fmaf(pv, kv[c], o[h][c]);
+        for (int c = 0; c < RC; c++)
+          o[h][c] = fmaf(pv.x, kv[0][c], fmaf(pv.y, kv[1][c], fmaf(pv.z, kv[2][c], fmaf(pv.w, kv[3][c], o[h][c]))));
       }
     }
     wave_sync();
   }
-  // merge the waves: every wave leaves (m, l, o) in its own LDS region
-  float* mg = (float*)wbase;                                       // [HB][r + 2]
+  // merge the waves: once all are done with the query and their tiles, every
+  // wave leaves (m, l, o) in its slice of the (re-used) LDS
+  __syncthreads();
+  const int MS = HB * (r + 2);
+  float* mg = (float*)smem + (size_t)wv * MS;                      // [HB][r + 2]
 #pragma unroll
   for (int h = 0; h < HB; h++) {
 #pragma unroll
@@ -276,43 +310,124 @@ __global__ void __launch_bounds__(256) latent_attn_k(const E* __restrict__ q_lat
     }
   }
   __syncthreads();
-  unsigned char* w0 = smem + (((size_t)HB * D * sizeof(float) + 15) & ~(size_t)15);
-  for (int i = threadIdx.x; i < nh * r; i += blockDim.x) {
-    const int h = i / r, c = i - h * r;
+  const float* m0 = (const float*)smem;
+  for (int i = threadIdx.x; i < nh * (r + 2); i += blockDim.x) {
+    const int h = i / (r + 2), c = i - h * (r + 2);
     float M = -INFINITY;
-    for (int w = 0; w < NW; w++) M = fmaxf(M, ((const float*)(w0 + w * wave_bytes))[h * (r + 2) + r]);
+    for (int w = 0; w < NW; w++) M = fmaxf(M, m0[(size_t)w * MS + h * (r + 2) + r]);
     float L = 0.f, O = 0.f;
     for (int w = 0; w < NW; w++) {
-      const float* g = (const float*)(w0 + w * wave_bytes) + h * (r + 2);
+      const float* g = m0 + (size_t)w * MS + h * (r + 2);
       const float mw = g[r];
       const float f = mw == -INFINITY ? 0.f : expf(mw - M);
       L += g[r + 1] * f;
-      O += g[c] * f;
+      if (c < r) O += g[c] * f;
     }
-    float v = O / L;
-    if (gate) v *= 1.0f / (1.0f + expf(-ldf(gate + (int64_t)t * g_st + h0 + h)));
-    stf(out + ((int64_t)t * H + h0 + h) * r + c, v);
+    if (nsplit > 1) {                                              // partial (o, m, l) of this key split
+      float* pp = part + (((int64_t)t * H + h0 + h) * nsplit + zs) * (r + 2);
+      pp[c] = c < r ? O : (c == r ? M : L);
+    } else if (c < r) {
+      float v = O / L;
+      if (gate) v *= 1.0f / (1.0f + expf(-ldf(gate + (int64_t)t * g_st + h0 + h)));
+      stf(out + ((int64_t)t * H + h0 + h) * r + c, v);
+    }
+  }
+}
+
+// merge of the key splits: part [T, H, nsplit, r + 2] -> out [T, H, r]
+template <typename E>
+__global__ void __launch_bounds__(128) latent_attn_combine_k(const float* __restrict__ part, const E* __restrict__ gate,
+                                                            int64_t g_st, E* __restrict__ out, int H, int r,
+                                                            int nsplit) {
+  const int64_t t = blockIdx.x;
+  const int h = blockIdx.y;
+  const float* pp = part + ((t * H + h) * nsplit) * (int64_t)(r + 2);
+  float M = -INFINITY;
+  for (int z = 0; z < nsplit; z++) M = fmaxf(M, pp[(int64_t)z * (r + 2) + r]);
+  float L = 0.f;
+  for (int z = 0; z < nsplit; z++) {
+    const float mz = pp[(int64_t)z * (r + 2) + r];
+    L += mz == -INFINITY ? 0.f : pp[(int64_t)z * (r + 2) + r + 1] * expf(mz - M);
+  }
+  const float g = gate ? 1.0f / (1.0f + expf(-ldf(gate + t * g_st + h))) : 1.0f;
+  for (int c = threadIdx.x; c < r; c += blockDim.x) {
+    float O = 0.f;
+    for (int z = 0; z < nsplit; z++) {
+      const float mz = pp[(int64_t)z * (r + 2) + r];
+      if (mz != -INFINITY) O += pp[(int64_t)z * (r + 2) + c] * expf(mz - M);
+    }
+    stf(out + (t * H + h) * r + c, O / L * g);
+  }
+}
+
+// Causal softmax over f32 score rows (the library-GEMM prefill path): row i
+// belongs to query token i / H at position pos[i / H]; keys j <= pos get
+// softmax(scale * s) in f32, the others 0.  E = float: written in place.
+// E = bf16: the f32 weight leaves as a pair of bf16 values hi + lo (hi the
+// rounded weight, lo the rounded remainder), so the following bf16 products
+// carry the weights to ~2^-17 instead of 2^-9.
+template <typename E>
+__global__ void __launch_bounds__(256) causal_softmax_k(float* __restrict__ sc, int64_t ld, const int64_t* __restrict__ pos,
+                                                       int H, float scale, int L, E* __restrict__ hi, E* __restrict__ lo) {
+  __shared__ float red[16];
+  const int64_t row = blockIdx.x;
+  const int64_t p = pos[row / H];
+  const int nk = (int)min((int64_t)L, p + 1);
+  float* s = sc + row * ld;
+  float mx = -INFINITY;
+  for (int j = threadIdx.x; j < nk; j += blockDim.x) mx = fmaxf(mx, s[j] * scale);
+  mx = wave_max(mx);
+  __syncthreads();
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = mx;
+  __syncthreads();
+  for (int i = 0; i < (int)(blockDim.x >> 6); i++) mx = fmaxf(mx, red[i]);
+  float sum = 0.f;
+  for (int j = threadIdx.x; j < nk; j += blockDim.x) {
+    const float e = expf(s[j] * scale - mx);
+    s[j] = e;
+    sum += e;
+  }
+  const float inv = 1.0f / block_sum(sum, red);
+  for (int j = threadIdx.x; j < L; j += blockDim.x) {
+    const float w = j < nk ? s[j] * inv : 0.f;
+    if (hi) {
+      const E h = (E)w;
+      hi[row * ld + j] = h;
+      lo[row * ld + j] = (E)(w - (float)h);
+    } else {
+      s[j] = w;
+    }
   }
 }
 
 // ------------------------------------------------------------------ mLSTM
-// One wave: 64 value columns of one (sequence, head).  S [d][64] lives in LDS
-// column-per-lane; n [d] is kept redundantly by every column block.
-template <typename E>
-__global__ void __launch_bounds__(64) mlstm_scan_k(const E* __restrict__ q, int64_t q_ld, const E* __restrict__ k,
-                                                  int64_t k_ld, const E* __restrict__ v, int64_t v_ld,
-                                                  const E* __restrict__ ipre, int64_t i_ld, const E* __restrict__ fpre,
-                                                  int64_t f_ld, const float* __restrict__ ib, const float* __restrict__ fb,
-                                                  float cap, float* __restrict__ Sg, float* __restrict__ ng,
-                                                  float* __restrict__ mgl, const int32_t* __restrict__ cu,
-                                                  const int32_t* __restrict__ slots, const int64_t* __restrict__ pos,
-                                                  float* __restrict__ out, int H, int d, int dv) {
+// One workgroup: 64 value columns of one (sequence, head).  Wave w keeps the
+// key rows [w DS, (w + 1) DS) of those columns in registers (the manner of
+// the RWKV-5 WKV kernel, misc.hip, with the key dimension split over up to
+// four waves).  Tokens go through LDS in chunks of TC: all threads stage q,
+// k, v and the gates; wave 0 runs the scalar recurrences (gates, running
+// maximum, normaliser n and its dot with q) once per chunk; every wave then
+// updates its rows and leaves a partial numerator per token; the partials are
+// summed in a fixed order, so a result never depends on how the tokens were
+// cut into steps.
+template <typename E, int DS>
+__global__ void __launch_bounds__(256) mlstm_scan_k(const E* __restrict__ q, int64_t q_ld, const E* __restrict__ k,
+                                                   int64_t k_ld, const E* __restrict__ v, int64_t v_ld,
+                                                   const E* __restrict__ ipre, int64_t i_ld, const E* __restrict__ fpre,
+                                                   int64_t f_ld, const float* __restrict__ ib, const float* __restrict__ fb,
+                                                   float cap, float* __restrict__ Sg, float* __restrict__ ng,
+                                                   float* __restrict__ mgl, const int32_t* __restrict__ cu,
+                                                   const int32_t* __restrict__ slots, const int64_t* __restrict__ pos,
+                                                   float* __restrict__ out, int H, int d, int dv, int TC) {
   extern __shared__ __align__(16) unsigned char smem[];
-  float* S = (float*)smem;                 // [d][64]
-  float* nb = S + (size_t)d * 64;          // [d]
-  float* qb = nb + d;                      // [d]
-  float* kb = qb + d;                      // [d]
-  const int b = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6, NWV = blockDim.x >> 6, DP = NWV * DS;
+  float* qs = (float*)smem;                 // [TC][DP]
+  float* ks = qs + (size_t)TC * DP;         // [TC][DP]
+  float* vs = ks + (size_t)TC * DP;         // [TC][64]
+  float* part = vs + (size_t)TC * 64;       // [NWV][TC][64]
+  float* ab = part + (size_t)NWV * TC * 64; // a, b, den [3][TC]
+  float* gi = ab + 3 * TC;                  // log gates i, f [2][TC]
+  const int b = blockIdx.x, h = blockIdx.y;
   const int j = blockIdx.z * 64 + lane;
   const bool jv = j < dv;
   const int t0 = cu[b], t1 = cu[b + 1];
@@ -321,46 +436,94 @@ __global__ void __launch_bounds__(64) mlstm_scan_k(const E* __restrict__ q, int6
   const bool fresh = pos[t0] == 0;
   float* Ss = Sg + ((slot * H + h) * d) * (int64_t)dv;
   float* ns = ng + (slot * H + h) * (int64_t)d;
-  float m = fresh ? 0.f : mgl[slot * H + h];
-  for (int dd = 0; dd < d; dd++) S[dd * 64 + lane] = (fresh || !jv) ? 0.f : Ss[(int64_t)dd * dv + j];
-  for (int dd = lane; dd < d; dd += 64) nb[dd] = fresh ? 0.f : ns[dd];
-  const float qscale = 1.0f / sqrtf((float)d);
-  for (int t = t0; t < t1; t++) {
-    __syncthreads();
-    for (int dd = lane; dd < d; dd += 64) {
-      qb[dd] = ldf(q + (int64_t)t * q_ld + h * d + dd) * qscale;
-      kb[dd] = ldf(k + (int64_t)t * k_ld + h * d + dd);
-    }
-    const float iz = (ldf(ipre + (int64_t)t * i_ld + h) + ib[h]) / cap;
-    const float fz = cap * tanhf((ldf(fpre + (int64_t)t * f_ld + h) + fb[h]) / cap);
-    const float ig = cap * tanhf(iz);
-    const float fg = fminf(fz, 0.f) - log1pf(expf(-fabsf(fz)));    // logsigmoid
-    const float mn = fmaxf(fg + m, ig);
-    const float a = expf(fg + m - mn), bb = expf(ig - mn);
-    m = mn;
-    const float vj = jv ? ldf(v + (int64_t)t * v_ld + h * dv + j) : 0.f;
-    __syncthreads();
-    float acc = 0.f;
-    for (int dd = 0; dd < d; dd++) {
-      const float s = a * S[dd * 64 + lane] + (bb * kb[dd]) * vj;
-      S[dd * 64 + lane] = s;
-      acc = fmaf(s, qb[dd], acc);
-    }
-    float part = 0.f;
-    for (int dd = lane; dd < d; dd += 64) {
-      const float nn = a * nb[dd] + bb * kb[dd];
-      nb[dd] = nn;
-      part = fmaf(nn, qb[dd], part);
-    }
-    const float nq = wave_sum(part);
-    const float den = fmaxf(fabsf(nq), expf(-m)) + 1e-6f;
-    if (jv) out[((int64_t)t * H + h) * dv + j] = acc / den;
+  float s[DS];
+#pragma unroll
+  for (int i = 0; i < DS; i++) {
+    const int row = w * DS + i;
+    s[i] = (fresh || !jv || row >= d) ? 0.f : Ss[(int64_t)row * dv + j];
   }
-  __syncthreads();
-  if (jv)
-    for (int dd = 0; dd < d; dd++) Ss[(int64_t)dd * dv + j] = S[dd * 64 + lane];
-  if (blockIdx.z == 0) {
-    for (int dd = lane; dd < d; dd += 64) ns[dd] = nb[dd];
+  float nreg[4] = {0.f, 0.f, 0.f, 0.f};
+  float m = 0.f;
+  if (w == 0 && !fresh) {
+    m = mgl[slot * H + h];
+#pragma unroll
+    for (int c = 0; c < 4; c++)
+      if (lane + 64 * c < d) nreg[c] = ns[lane + 64 * c];
+  }
+  const float qscale = 1.0f / sqrtf((float)d);
+  for (int tb = t0; tb < t1; tb += TC) {
+    const int nt = min(TC, t1 - tb);
+    __syncthreads();
+    for (int i = threadIdx.x; i < nt * DP; i += blockDim.x) {
+      const int tt = i / DP, c = i - tt * DP;
+      qs[i] = c < d ? ldf(q + (int64_t)(tb + tt) * q_ld + h * d + c) * qscale : 0.f;
+      ks[i] = c < d ? ldf(k + (int64_t)(tb + tt) * k_ld + h * d + c) : 0.f;
+    }
+    for (int i = threadIdx.x; i < nt * 64; i += blockDim.x) {
+      const int tt = i >> 6, col = blockIdx.z * 64 + (i & 63);
+      vs[i] = col < dv ? ldf(v + (int64_t)(tb + tt) * v_ld + h * dv + col) : 0.f;
+    }
+    for (int tt = threadIdx.x; tt < nt; tt += blockDim.x) {
+      const float iz = (ldf(ipre + (int64_t)(tb + tt) * i_ld + h) + ib[h]) / cap;
+      const float fz = cap * tanhf((ldf(fpre + (int64_t)(tb + tt) * f_ld + h) + fb[h]) / cap);
+      gi[tt] = cap * tanhf(iz);
+      gi[TC + tt] = fminf(fz, 0.f) - log1pf(expf(-fabsf(fz)));     // logsigmoid
+    }
+    __syncthreads();
+    if (w == 0) {
+      for (int tt = 0; tt < nt; tt++) {
+        const float ig = gi[tt], fg = gi[TC + tt];
+        const float mn = fmaxf(fg + m, ig);
+        const float a = expf(fg + m - mn), bb = expf(ig - mn);
+        m = mn;
+        float pq = 0.f;
+#pragma unroll
+        for (int c = 0; c < 4; c++) {
+          const int row = lane + 64 * c;
+          if (row < DP) {
+            nreg[c] = a * nreg[c] + bb * ks[tt * DP + row];
+            pq = fmaf(nreg[c], qs[tt * DP + row], pq);
+          }
+        }
+        const float nq = wave_sum(pq);
+        if (lane == 0) {
+          ab[tt] = a;
+          ab[TC + tt] = bb;
+          ab[2 * TC + tt] = fmaxf(fabsf(nq), expf(-m)) + 1e-6f;
+        }
+      }
+    }
+    __syncthreads();
+    for (int tt = 0; tt < nt; tt++) {
+      const float a = ab[tt], bb = ab[TC + tt], vj = vs[tt * 64 + lane];
+      const float* kk = ks + tt * DP + w * DS;
+      const float* qq = qs + tt * DP + w * DS;
+      float acc = 0.f;
+#pragma unroll
+      for (int i = 0; i < DS; i++) {
+        s[i] = fmaf(a, s[i], (bb * kk[i]) * vj);
+        acc = fmaf(s[i], qq[i], acc);
+      }
+      part[((size_t)w * TC + tt) * 64 + lane] = acc;
+    }
+    __syncthreads();
+    for (int tt = w; tt < nt; tt += NWV) {
+      float sum = 0.f;
+      for (int ww = 0; ww < NWV; ww++) sum += part[((size_t)ww * TC + tt) * 64 + lane];
+      if (jv) out[((int64_t)(tb + tt) * H + h) * dv + j] = sum / ab[2 * TC + tt];
+    }
+  }
+  if (jv) {
+#pragma unroll
+    for (int i = 0; i < DS; i++) {
+      const int row = w * DS + i;
+      if (row < d) Ss[(int64_t)row * dv + j] = s[i];
+    }
+  }
+  if (w == 0 && blockIdx.z == 0) {
+#pragma unroll
+    for (int c = 0; c < 4; c++)
+      if (lane + 64 * c < d) ns[lane + 64 * c] = nreg[c];
     if (lane == 0) mgl[slot * H + h] = m;
   }
 }
@@ -437,63 +600,110 @@ void latent_kv_store(bool bf16, const void* dkv, int64_t ld, const void* norm_w,
                                        num_rows));
 }
 
-static int pad_row(int D, int esz) {
-  // row stride (elements) whose dword stride is odd: lanes reading one column of 64 rows hit 64 banks
-  if (esz == 4) return (D & 1) ? D : D + 1;
-  int dp = (D + 1) & ~1;                   // even element count -> whole dwords
-  return ((dp / 2) & 1) ? dp : dp + 2;
+static int pad_row(int D) {
+  // row stride (elements) = 4 (mod 8): 4-element reads of a column group by 64 lanes spread over all banks
+  int dp = (D + 3) & ~3;
+  return (dp & 7) == 4 ? dp : dp + 4;
 }
 
-int latent_attention_plan(bool bf16, int H, int r, int dr, int* kt, int* nw) {
+// LDS plan: heads per workgroup, keys per tile, waves.  The tile buffers, the
+// query block and (afterwards, over the same memory) the waves' merge slices
+// must fit in 64 KB.
+int latent_attention_plan(bool bf16, int H, int r, int dr, int* kt, int* nw, int* hbo) {
   const int esz = bf16 ? 2 : 4, D = r + dr;
-  const int DP = pad_row(D, esz);
-  const size_t qbytes = ((size_t)HB * D * 4 + 15) & ~(size_t)15;
+  const int DP = pad_row(D), D4 = (D + 3) & ~3;
   static const int opts[][2] = {{64, 4}, {64, 2}, {32, 4}, {32, 2}, {64, 1}, {16, 4}, {32, 1}, {16, 2}, {16, 1}};
-  for (auto& o : opts) {
-    const size_t wave = ((size_t)o[0] * DP * esz + (size_t)HB * o[0] * 4 + 15) & ~(size_t)15;
-    if (wave < (size_t)HB * (r + 2) * 4) continue;
-    const size_t total = qbytes + wave * o[1];
-    if (total <= 64 * 1024) {
-      *kt = o[0];
-      *nw = o[1];
-      return (int)total;
+  // 16 heads per workgroup only while the f32 accumulators (heads x latent columns per lane) stay in registers
+  for (int hb = (H > 8 && r <= 128) ? 16 : 8; hb >= 8; hb -= 8) {
+    const size_t qbytes = ((size_t)hb * D4 * esz + 15) & ~(size_t)15;
+    for (auto& o : opts) {
+      const size_t wave = ((size_t)o[0] * DP * esz + (size_t)hb * o[0] * 4 + 15) & ~(size_t)15;
+      const size_t total = qbytes + wave * o[1];
+      if (total <= 64 * 1024 && (size_t)o[1] * hb * (r + 2) * 4 <= total) {
+        *kt = o[0];
+        *nw = o[1];
+        *hbo = hb;
+        return (int)total;
+      }
     }
   }
   return -1;
 }
 
+int latent_attention_splits(bool bf16, int T, int H, int r, int dr, int max_ctx) {
+  int KT = 0, NW = 0, hb = 8;
+  if (latent_attention_plan(bf16, H, r, dr, &KT, &NW, &hb) < 0) return 1;
+  const int64_t blocks = (int64_t)T * ((H + hb - 1) / hb);
+  const int tiles = (max_ctx + KT - 1) / KT;
+  int ns = (int)((1024 + blocks - 1) / blocks);            // ~4 workgroups per CU
+  ns = ns > (tiles + NW - 1) / NW ? (tiles + NW - 1) / NW : ns;
+  return ns < 1 ? 1 : (ns > 64 ? 64 : ns);
+}
+
 void latent_attention(bool bf16, const void* q_lat, const void* q_rot, int64_t qr_st, int64_t qr_sh, const void* rows,
                       int bs, const int32_t* block_tables, int bt_width, const int32_t* seq_of, const int64_t* pos,
-                      float scale, const void* gate, int64_t g_st, void* out, int T, int H, int r, int dr,
-                      hipStream_t st) {
+                      float scale, const void* gate, int64_t g_st, void* out, float* part, int nsplit, int T, int H,
+                      int r, int dr, hipStream_t st) {
   if (T <= 0) return;
-  int KT = 0, NW = 0;
-  const int lds = latent_attention_plan(bf16, H, r, dr, &KT, &NW);
+  int KT = 0, NW = 0, hb = 8;
+  const int lds = latent_attention_plan(bf16, H, r, dr, &KT, &NW, &hb);
   if (lds < 0) return;                     // refused by the caller beforehand
-  const int DP = pad_row(r + dr, bf16 ? 2 : 4);
+  const int DP = pad_row(r + dr);
   const int rc = (r + 63) / 64;
-  dim3 grid(T, (H + HB - 1) / HB), block(64 * NW);
-#define SM_ATTN(RC)                                                                                                  \
-  SM_DISPATCH(bf16, hipLaunchKernelGGL((latent_attn_k<E, RC>), grid, block, lds, st, (const E*)q_lat, (const E*)q_rot, \
-                                       qr_st, qr_sh, (const E*)rows, bs, block_tables, bt_width, seq_of, pos, scale,   \
-                                       (const E*)gate, g_st, (E*)out, H, r, dr, KT, DP))
-  if (rc <= 1) { SM_ATTN(1); }
-  else if (rc <= 2) { SM_ATTN(2); }
-  else if (rc <= 4) { SM_ATTN(4); }
-  else { SM_ATTN(8); }
+  dim3 grid(T, (H + hb - 1) / hb, nsplit), block(64 * NW);
+#define SM_ATTN(RC, HBV)                                                                                              \
+  SM_DISPATCH(bf16, hipLaunchKernelGGL((latent_attn_k<E, RC, HBV>), grid, block, lds, st, (const E*)q_lat,             \
+                                       (const E*)q_rot, qr_st, qr_sh, (const E*)rows, bs, block_tables, bt_width,      \
+                                       seq_of, pos, scale, (const E*)gate, g_st, (E*)out, part, H, r, dr, KT, DP))
+  if (hb == 8) {
+    if (rc <= 1) { SM_ATTN(1, 8); }
+    else if (rc <= 2) { SM_ATTN(2, 8); }
+    else if (rc <= 4) { SM_ATTN(4, 8); }
+    else { SM_ATTN(8, 8); }
+  } else {
+    if (rc <= 1) { SM_ATTN(1, 16); }
+    else if (rc <= 2) { SM_ATTN(2, 16); }
+    else if (rc <= 4) { SM_ATTN(4, 16); }
+    else { SM_ATTN(8, 16); }
+  }
 #undef SM_ATTN
+  if (nsplit > 1) {
+    SM_DISPATCH(bf16, hipLaunchKernelGGL(latent_attn_combine_k<E>, dim3(T, H), dim3(128), 0, st, part, (const E*)gate,
+                                         g_st, (E*)out, H, r, nsplit));
+  }
+}
+
+void causal_softmax(bool bf16, float* sc, int64_t ld, const int64_t* pos, int H, float scale, int64_t R, int L, void* hi,
+                    void* lo, hipStream_t st) {
+  if (R <= 0 || L <= 0) return;
+  if (bf16) {
+    hipLaunchKernelGGL(causal_softmax_k<__bf16>, dim3((unsigned)R), dim3(256), 0, st, sc, ld, pos, H, scale, L,
+                       (__bf16*)hi, (__bf16*)lo);
+  } else {
+    hipLaunchKernelGGL(causal_softmax_k<float>, dim3((unsigned)R), dim3(256), 0, st, sc, ld, pos, H, scale, L,
+                       (float*)nullptr, (float*)nullptr);
+  }
 }
 
 void mlstm_scan(bool bf16, const void* q, int64_t q_ld, const void* k, int64_t k_ld, const void* v, int64_t v_ld,
                 const void* ipre, int64_t i_ld, const void* fpre, int64_t f_ld, const float* ib, const float* fb,
                 float cap, float* S, float* n, float* m, const int32_t* cu, const int32_t* slots, const int64_t* pos,
                 float* out, int B, int H, int d, int dv, hipStream_t st) {
-  if (B <= 0) return;
-  const size_t lds = ((size_t)d * 64 + 3 * (size_t)d) * 4;
-  dim3 grid(B, H, (dv + 63) / 64);
-  SM_DISPATCH(bf16, hipLaunchKernelGGL(mlstm_scan_k<E>, grid, dim3(64), lds, st, (const E*)q, q_ld, (const E*)k, k_ld,
-                                       (const E*)v, v_ld, (const E*)ipre, i_ld, (const E*)fpre, f_ld, ib, fb, cap, S, n,
-                                       m, cu, slots, pos, out, H, d, dv));
+  if (B <= 0 || d > 256) return;           // d checked by the caller
+  const int DS = d <= 32 ? 8 : d <= 64 ? 16 : d <= 128 ? 32 : 64;
+  const int NWV = (d + DS - 1) / DS, DP = NWV * DS;
+  const int TC = 16;                       // tokens staged per chunk (52 KB of LDS at d = 256)
+  const size_t lds = ((size_t)2 * TC * DP + (size_t)TC * 64 + (size_t)NWV * TC * 64 + 5 * (size_t)TC) * 4;
+  dim3 grid(B, H, (dv + 63) / 64), block(64 * NWV);
+#define SM_SCAN(DSV)                                                                                                  \
+  SM_DISPATCH(bf16, hipLaunchKernelGGL((mlstm_scan_k<E, DSV>), grid, block, lds, st, (const E*)q, q_ld, (const E*)k,   \
+                                       k_ld, (const E*)v, v_ld, (const E*)ipre, i_ld, (const E*)fpre, f_ld, ib, fb,    \
+                                       cap, S, n, m, cu, slots, pos, out, H, d, dv, TC))
+  if (DS == 8) { SM_SCAN(8); }
+  else if (DS == 16) { SM_SCAN(16); }
+  else if (DS == 32) { SM_SCAN(32); }
+  else { SM_SCAN(64); }
+#undef SM_SCAN
 }
 
 void head_rms_gate(bool bf16, const float* h, const void* norm_w, const void* gate, int64_t g_ld, void* out, int T,

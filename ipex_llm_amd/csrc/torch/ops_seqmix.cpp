@@ -138,15 +138,39 @@ Tensor sm_latent_attention(const Tensor& q_lat, const Tensor& q_rot, const Tenso
     gp = gate->data_ptr();
     gst = gate->stride(0);
   }
-  int kt = 0, nw = 0;
-  TORCH_CHECK(illm::sm::latent_attention_plan(bf(q_lat), (int)H, (int)r, (int)dr, &kt, &nw) > 0,
+  int kt = 0, nw = 0, hb = 0;
+  TORCH_CHECK(illm::sm::latent_attention_plan(bf(q_lat), (int)H, (int)r, (int)dr, &kt, &nw, &hb) > 0,
               "sm_latent_attention: a key tile of r + dr = ", r + dr, " does not fit in LDS");
   Tensor out = at::empty({T, H, r}, q_lat.options());
+  if (T == 0) return out;
+  const int nsplit = illm::sm::latent_attention_splits(bf(q_lat), (int)T, (int)H, (int)r, (int)dr, (int)max_ctx);
+  Tensor part;
+  if (nsplit > 1) part = at::empty({T, H, nsplit, r + 2}, q_lat.options().dtype(at::kFloat));
   illm::sm::latent_attention(bf(q_lat), q_lat.data_ptr(), q_rot.data_ptr(), q_rot.stride(0), q_rot.stride(1),
                              rows.data_ptr(), (int)rows.size(1), block_tables.data_ptr<int32_t>(),
                              (int)block_tables.size(1), seq_of.data_ptr<int32_t>(), pos.data_ptr<int64_t>(), (float)scale,
-                             gp, gst, out.data_ptr(), (int)T, (int)H, (int)r, (int)dr, stream());
+                             gp, gst, out.data_ptr(), nsplit > 1 ? part.data_ptr<float>() : nullptr, nsplit, (int)T,
+                             (int)H, (int)r, (int)dr, stream());
   return out;
+}
+
+// scores f32 [R, L] (R = tokens x H rows) -> causal softmax weights; bf16 pair (hi, lo) or in place (f32)
+std::tuple<Tensor, Tensor> sm_causal_softmax(Tensor& scores, const Tensor& pos, int64_t H, double scale, bool act_f32) {
+  c10::DeviceGuard g(scores.device());
+  TORCH_CHECK(scores.is_cuda() && scores.dim() == 2 && scores.scalar_type() == at::kFloat && scores.is_contiguous(),
+              "sm_causal_softmax: scores f32 [R, L] contiguous");
+  const int64_t R = scores.size(0), L = scores.size(1);
+  TORCH_CHECK(H >= 1 && R % H == 0, "sm_causal_softmax: rows must be tokens x heads");
+  check_idx(pos, at::kLong, R / H, "sm_causal_softmax: pos int64 [R / H]");
+  Tensor hi, lo;
+  if (!act_f32) {
+    hi = at::empty({R, L}, scores.options().dtype(at::kBFloat16));
+    lo = at::empty({R, L}, scores.options().dtype(at::kBFloat16));
+  }
+  illm::sm::causal_softmax(!act_f32, scores.data_ptr<float>(), L, pos.data_ptr<int64_t>(), (int)H, (float)scale, R, (int)L,
+                           act_f32 ? nullptr : hi.data_ptr(), act_f32 ? nullptr : lo.data_ptr(), stream());
+  if (act_f32) return {scores, scores};
+  return {hi, lo};
 }
 
 Tensor sm_mlstm_scan(const Tensor& q, const Tensor& k, const Tensor& v, const Tensor& ipre, const Tensor& fpre,
@@ -176,7 +200,7 @@ Tensor sm_mlstm_scan(const Tensor& q, const Tensor& k, const Tensor& v, const Te
                   m.scalar_type() == at::kFloat && m.is_contiguous() && m.dim() == 2 && m.size(0) == S.size(0) &&
                   m.size(1) == H,
               "sm_mlstm_scan: state S [slots, H, d, dv], n [slots, H, d], m [slots, H] f32");
-  TORCH_CHECK(d >= 1 && (d * 64 + 3 * d) * 4 <= 64 * 1024, "sm_mlstm_scan: key size too large for the LDS-resident state");
+  TORCH_CHECK(d >= 1 && d <= 256, "sm_mlstm_scan: key size per head must be 1..256 (register-resident state rows)");
   TORCH_CHECK(max_q >= 0 && max_q <= T, "sm_mlstm_scan: max_q");
   Tensor out = at::empty({T, H, dv}, q.options().dtype(at::kFloat));
   if (T == 0 || B == 0) return out;
@@ -228,6 +252,7 @@ TORCH_LIBRARY_FRAGMENT(ipex_llm_amd, m) {
         "float scale, Tensor? gate, int max_ctx, bool act_f32) -> Tensor");
   m.def("sm_mlstm_scan(Tensor q, Tensor k, Tensor v, Tensor ipre, Tensor fpre, Tensor ib, Tensor fb, float cap, "
         "Tensor(a!) S, Tensor(b!) n, Tensor(c!) m, Tensor cu, Tensor slots, Tensor pos, int max_q) -> Tensor");
+  m.def("sm_causal_softmax(Tensor(a!) scores, Tensor pos, int H, float scale, bool act_f32) -> (Tensor, Tensor)");
   m.def("sm_head_rms_gate(Tensor h, Tensor norm_w, Tensor gate, float eps, bool act_f32) -> Tensor");
   m.def("sm_glu_gelu(Tensor gu) -> Tensor");
 }
@@ -240,6 +265,7 @@ TORCH_LIBRARY_IMPL(ipex_llm_amd, CUDA, m) {
   m.impl("sm_latent_kv_store", &sm_latent_kv_store);
   m.impl("sm_latent_attention", &sm_latent_attention);
   m.impl("sm_mlstm_scan", &sm_mlstm_scan);
+  m.impl("sm_causal_softmax", &sm_causal_softmax);
   m.impl("sm_head_rms_gate", &sm_head_rms_gate);
   m.impl("sm_glu_gelu", &sm_glu_gelu);
 }

@@ -314,7 +314,8 @@ class NativeCausalLM(nn.Module):
         from .cache import PagedKVCache
         s = self.spec
         nblk = num_blocks or batch * ((max_tokens + block_size - 1) // block_size)
-        self.ensure_rope_cache(max_tokens + 1)
+        # (whole blocks: a captured decode step warms up at the last slots of the allocation)
+        self.ensure_rope_cache(((max_tokens + block_size - 1) // block_size) * block_size + 1)
         cache = PagedKVCache(len(self.layers), nblk, s.num_kv_heads, s.head_dim, block_size, self.dtype,
                              self.device, kv_fp8)
         if any(L.self_attn.lf is not None for L in self.layers):

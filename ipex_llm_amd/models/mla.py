@@ -93,7 +93,9 @@ class MLACausalLM(NativeCausalLM):
                    num_blocks: Optional[int] = None):
         from .cache import BlockAllocator, PagedKVCache
         nblk = num_blocks or batch * ((max_tokens + block_size - 1) // block_size)
-        self.ensure_rope_cache(max_tokens + 1)
+        # whole blocks: the decode step's capture warm-up runs at the last slots of a
+        # sequence's allocation, and the rotary rows are gathered by position
+        self.ensure_rope_cache(((max_tokens + block_size - 1) // block_size) * block_size + 1)
         c = PagedKVCache.__new__(PagedKVCache)
         c.num_layers, c.num_blocks = len(self.layers), nblk
         c.Hkv, c.D, c.bs = 1, self.r + self.dr, block_size

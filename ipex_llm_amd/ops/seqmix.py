@@ -157,8 +157,8 @@ def latent_attention(q_lat: torch.Tensor, q_rot: torch.Tensor, rows: torch.Tenso
     count and key count."""
     T, H, r = q_lat.shape
     if native(q_lat):
-        return _ops().sm_latent_attention(q_lat.contiguous(), q_rot, rows, block_tables, seq_of, pos, float(scale),
-                                          gate, max(ctx_lens), out_dtype == torch.float32)
+        return _latent_attention_gpu(q_lat, q_rot, rows, block_tables, seq_of, pos, float(scale), gate, q_lens,
+                                     ctx_lens, out_dtype)
     out = torch.empty(T, H, r, dtype=torch.float32, device=q_lat.device)
     bs = rows.shape[1]
     t0 = 0
@@ -177,6 +177,84 @@ def latent_attention(q_lat: torch.Tensor, q_rot: torch.Tensor, rows: torch.Tenso
     if gate is not None:
         out = out * torch.sigmoid(gate.float())[..., None]
     return out.to(out_dtype)
+
+
+# Portions of at least this many tokens take the library-GEMM path on the GPU:
+# scores and the weighted sum of latents are GEMM-shaped ([tokens x heads, r + dr]
+# x [r + dr, keys] and [tokens x heads, keys] x [keys, r]) and go to the vendor
+# GEMM with f32 results (as models/mla.py does for its latent attention), with
+# the fused causal softmax kernel between them.  Shorter portions and decoded
+# tokens run the one-pass flash kernel, which keeps everything in f32 registers.
+GEMM_MIN_Q = int(__import__("os").environ.get("ILLM_LATENT_GEMM_MIN", "128"))
+GEMM_Q_BLOCK = int(__import__("os").environ.get("ILLM_LATENT_GEMM_BLOCK", "1024"))
+_mm_out_f32: Optional[bool] = None
+
+
+def _mm_f32(a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
+    """a @ b with an f32 result (16-bit operands: f32 accumulation, no rounding of the result)"""
+    global _mm_out_f32
+    if a.dtype == torch.float32:
+        return a @ b
+    if _mm_out_f32 is None:
+        try:
+            torch.mm(a[:16, :16].contiguous(), a[:16, :16].contiguous(), out_dtype=torch.float32)
+            _mm_out_f32 = True
+        except (TypeError, RuntimeError):
+            _mm_out_f32 = False
+    if _mm_out_f32:
+        return torch.mm(a, b, out_dtype=torch.float32)
+    return a.float() @ b.float()
+
+
+def _latent_attention_gemm(q_lat, q_rot, rows, table_row, pos, scale, L: int, n: int) -> torch.Tensor:
+    """one sequence's portion of n >= GEMM_MIN_Q tokens ending at key count L -> f32 [n, H, r]"""
+    _, H, r = q_lat.shape
+    bs = rows.shape[1]
+    nb = (L + bs - 1) // bs
+    kv = rows[table_row[:nb].long()].reshape(nb * bs, -1)           # this sequence's rows, in order
+    out = torch.empty(n, H, r, dtype=torch.float32, device=q_lat.device)
+    f32 = q_lat.dtype == torch.float32
+    for t0 in range(0, n, GEMM_Q_BLOCK):
+        t1 = min(n, t0 + GEMM_Q_BLOCK)
+        Lb = min(nb * bs, (L - n + t1 + 7) // 8 * 8)                 # keys the block's last token sees (rows past L: weight 0)
+        q2 = torch.cat([q_lat[t0:t1], q_rot[t0:t1]], -1).reshape((t1 - t0) * H, -1)
+        sc = _mm_f32(q2, kv[:Lb].t()).contiguous()
+        hi, lo = _ops().sm_causal_softmax(sc, pos[t0:t1].contiguous(), H, scale, f32)
+        c = kv[:Lb, :r]
+        o = _mm_f32(hi, c)
+        if not f32:
+            o += _mm_f32(lo, c)
+        out[t0:t1] = o.view(t1 - t0, H, r)
+    return out
+
+
+def _latent_attention_gpu(q_lat, q_rot, rows, block_tables, seq_of, pos, scale, gate, q_lens, ctx_lens, out_dtype):
+    T, H, r = q_lat.shape
+    f32 = out_dtype == torch.float32
+    big = [b for b, n in enumerate(q_lens) if n >= GEMM_MIN_Q]
+    if not big:
+        return _ops().sm_latent_attention(q_lat.contiguous(), q_rot, rows, block_tables, seq_of, pos, scale, gate,
+                                          max(ctx_lens), f32)
+    out = torch.empty(T, H, r, dtype=out_dtype, device=q_lat.device)
+    small, small_ctx, t0 = [], 1, 0
+    for b, (n, L) in enumerate(zip(q_lens, ctx_lens)):
+        if n >= GEMM_MIN_Q:
+            o = _latent_attention_gemm(q_lat[t0:t0 + n], q_rot[t0:t0 + n], rows, block_tables[b], pos[t0:t0 + n], scale,
+                                       L, n)
+            if gate is not None:
+                o = o * torch.sigmoid(gate[t0:t0 + n].float())[..., None]
+            out[t0:t0 + n] = o.to(out_dtype)
+        elif n:
+            small.append(torch.arange(t0, t0 + n, device=q_lat.device))
+            small_ctx = max(small_ctx, L)
+        t0 += n
+    if small:
+        idx = torch.cat(small)
+        o = _ops().sm_latent_attention(q_lat[idx].contiguous(), q_rot[idx], rows, block_tables,
+                                       seq_of[idx].contiguous(), pos[idx].contiguous(), scale,
+                                       gate[idx] if gate is not None else None, small_ctx, f32)
+        out[idx] = o
+    return out
 
 
 # ------------------------------------------------------------------ mLSTM
