@@ -190,6 +190,10 @@ template <> struct Ld4<__bf16> {
   }
 };
 
+template <typename E> struct Chunk4;
+template <> struct Chunk4<float> { typedef uint4 type; };
+template <> struct Chunk4<__bf16> { typedef uint2 type; };
+
 template <typename E, int RC, int HB>
 __global__ void __launch_bounds__(256) latent_attn_k(const E* __restrict__ q_lat, const E* __restrict__ q_rot,
                                                     int64_t qr_st, int64_t qr_sh, const E* __restrict__ rows, int bs,
@@ -210,13 +214,30 @@ __global__ void __launch_bounds__(256) latent_attn_k(const E* __restrict__ q_lat
   unsigned char* wbase = smem + q_bytes + wv * wave_bytes;
   E* kt = (E*)wbase;                                               // [KT][DP]
   float* pb = (float*)(wbase + (size_t)KT * DP * sizeof(E));       // [HB][KT]
-  for (int i = threadIdx.x; i < HB * D4; i += blockDim.x) {
-    const int h = i / D4, c = i - h * D4;
-    float v = 0.f;
-    if (h < nh && c < D)
-      v = c < r ? ldf(q_lat + ((int64_t)t * H + h0 + h) * r + c)
-                : ldf(q_rot + (int64_t)t * qr_st + (int64_t)(h0 + h) * qr_sh + (c - r));
-    stf(qs + i, v);
+  typedef typename Chunk4<E>::type C4;
+  if ((((int64_t)r | dr | qr_st | qr_sh) & 3) == 0 && ((uintptr_t)q_rot % sizeof(C4)) == 0) {
+    // whole 4-element chunks, every head's loads independent of the others (one latency, not HB x D)
+#pragma unroll
+    for (int h = 0; h < HB; h++) {
+      C4* dst = (C4*)(qs + h * D4);
+      if (h < nh) {
+        const C4* a = (const C4*)(q_lat + ((int64_t)t * H + h0 + h) * r);
+        const C4* b = (const C4*)(q_rot + (int64_t)t * qr_st + (int64_t)(h0 + h) * qr_sh);
+        for (int i = threadIdx.x; i < (r >> 2); i += blockDim.x) dst[i] = a[i];
+        for (int i = threadIdx.x; i < (dr >> 2); i += blockDim.x) dst[(r >> 2) + i] = b[i];
+      } else {
+        for (int i = threadIdx.x; i < D4; i += blockDim.x) stf(qs + h * D4 + i, 0.f);
+      }
+    }
+  } else {
+    for (int i = threadIdx.x; i < HB * D4; i += blockDim.x) {
+      const int h = i / D4, c = i - h * D4;
+      float v = 0.f;
+      if (h < nh && c < D)
+        v = c < r ? ldf(q_lat + ((int64_t)t * H + h0 + h) * r + c)
+                  : ldf(q_rot + (int64_t)t * qr_st + (int64_t)(h0 + h) * qr_sh + (c - r));
+      stf(qs + i, v);
+    }
   }
   // the whole tile buffer starts finite: rows and pad columns a tile does not fill are read with weight 0
   for (int i = lane; i < KT * DP; i += 64) stf(kt + i, 0.f);
@@ -237,18 +258,45 @@ __global__ void __launch_bounds__(256) latent_attn_k(const E* __restrict__ q_lat
     const int nvalid = (int)min((int64_t)KT, p - k0 + 1);
     const int64_t row0 = (int64_t)tab[k0 / bs] * bs + (k0 % bs);
     const E* src = rows + row0 * D;
-    for (int i = lane; i < nvalid * D; i += 64) {
-      const int j = i / D, c = i - j * D;
-      kt[j * DP + c] = src[i];
+    if ((D & 3) == 0) {
+      // 4-element chunks of the tile's contiguous rows; (row, column) advance without a division
+      const C4* s4 = (const C4*)src;
+      const int n4 = nvalid * (D >> 2);
+      int j = 0, c = lane * 4;
+      while (c >= D) { c -= D; j++; }
+      for (int i = lane; i < n4; i += 64 * 4) {
+        C4 v[4];
+        int jj[4], cc[4];
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+          jj[u] = j;
+          cc[u] = c;
+          if (i + 64 * u < n4) v[u] = s4[i + 64 * u];
+          c += 256;
+          while (c >= D) { c -= D; j++; }
+        }
+#pragma unroll
+        for (int u = 0; u < 4; u++)
+          if (i + 64 * u < n4) *(C4*)(kt + jj[u] * DP + cc[u]) = v[u];
+      }
+    } else {
+      for (int i = lane; i < nvalid * D; i += 64) {
+        const int j = i / D, c = i - j * D;
+        kt[j * DP + c] = src[i];
+      }
     }
     wave_sync();                                                   // the tile is in LDS
     float s[HB];
 #pragma unroll
     for (int h = 0; h < HB; h++) s[h] = 0.f;
-    const bool valid = lane < nvalid;
+    // 64 / KT lanes share a key: each takes a slice of the r + dr products, summed by lane exchange
+    const int kj = lane & (KT - 1), grp = lane / KT, G = 64 / KT;
+    const bool valid = kj < nvalid;
     if (valid) {
-      const E* kr = kt + lane * DP;
-      for (int c = 0; c < D4; c += 4) {
+      const E* kr = kt + kj * DP;
+      const int steps = D4 >> 2;
+      for (int c4 = grp * steps / G; c4 < (grp + 1) * steps / G; c4++) {
+        const int c = c4 * 4;
         float kv[4];
         Ld4<E>::get(kr + c, kv);
 #pragma unroll
@@ -259,13 +307,17 @@ __global__ void __launch_bounds__(256) latent_attn_k(const E* __restrict__ q_lat
         }
       }
     }
+    for (int off = KT; off < 64; off <<= 1) {
+#pragma unroll
+      for (int h = 0; h < HB; h++) s[h] += __shfl_xor(s[h], off, 64);
+    }
 #pragma unroll
     for (int h = 0; h < HB; h++) {
       const float sv = valid ? s[h] * scale : -INFINITY;
       const float mn = fmaxf(m[h], wave_max(sv));
       const float alpha = m[h] == -INFINITY ? 0.f : expf(m[h] - mn);
       const float pv = valid ? expf(sv - mn) : 0.f;
-      l[h] = l[h] * alpha + wave_sum(pv);
+      l[h] = l[h] * alpha + wave_sum(lane < KT ? pv : 0.f);
       m[h] = mn;
 #pragma unroll
       for (int c = 0; c < RC; c++) o[h][c] *= alpha;
@@ -339,24 +391,24 @@ template <typename E>
 __global__ void __launch_bounds__(128) latent_attn_combine_k(const float* __restrict__ part, const E* __restrict__ gate,
                                                             int64_t g_st, E* __restrict__ out, int H, int r,
                                                             int nsplit) {
+  __shared__ float wz[64];                                          // exp(m_z - M) / L * gate, nsplit <= 64
   const int64_t t = blockIdx.x;
   const int h = blockIdx.y;
   const float* pp = part + ((t * H + h) * nsplit) * (int64_t)(r + 2);
-  float M = -INFINITY;
-  for (int z = 0; z < nsplit; z++) M = fmaxf(M, pp[(int64_t)z * (r + 2) + r]);
-  float L = 0.f;
-  for (int z = 0; z < nsplit; z++) {
-    const float mz = pp[(int64_t)z * (r + 2) + r];
-    L += mz == -INFINITY ? 0.f : pp[(int64_t)z * (r + 2) + r + 1] * expf(mz - M);
+  if (threadIdx.x < 64) {
+    const int z = threadIdx.x;
+    const float mz = z < nsplit ? pp[(int64_t)z * (r + 2) + r] : -INFINITY;
+    const float M = wave_max(mz);
+    const float e = mz == -INFINITY ? 0.f : expf(mz - M);
+    const float L = wave_sum(z < nsplit ? pp[(int64_t)z * (r + 2) + r + 1] * e : 0.f);
+    const float g = gate ? 1.0f / (1.0f + expf(-ldf(gate + t * g_st + h))) : 1.0f;
+    wz[z] = e / L * g;
   }
-  const float g = gate ? 1.0f / (1.0f + expf(-ldf(gate + t * g_st + h))) : 1.0f;
+  __syncthreads();
   for (int c = threadIdx.x; c < r; c += blockDim.x) {
     float O = 0.f;
-    for (int z = 0; z < nsplit; z++) {
-      const float mz = pp[(int64_t)z * (r + 2) + r];
-      if (mz != -INFINITY) O += pp[(int64_t)z * (r + 2) + c] * expf(mz - M);
-    }
-    stf(out + (t * H + h) * r + c, O / L * g);
+    for (int z = 0; z < nsplit; z++) O = fmaf(pp[(int64_t)z * (r + 2) + c], wz[z], O);
+    stf(out + (t * H + h) * r + c, O);
   }
 }
 
@@ -418,7 +470,7 @@ __global__ void __launch_bounds__(256) mlstm_scan_k(const E* __restrict__ q, int
                                                    float cap, float* __restrict__ Sg, float* __restrict__ ng,
                                                    float* __restrict__ mgl, const int32_t* __restrict__ cu,
                                                    const int32_t* __restrict__ slots, const int64_t* __restrict__ pos,
-                                                   float* __restrict__ out, int H, int d, int dv, int TC) {
+                                                   float* __restrict__ out, int H, int d, int dv, int TC, bool vec) {
   extern __shared__ __align__(16) unsigned char smem[];
   const int lane = threadIdx.x & 63, w = threadIdx.x >> 6, NWV = blockDim.x >> 6, DP = NWV * DS;
   float* qs = (float*)smem;                 // [TC][DP]
@@ -454,14 +506,63 @@ __global__ void __launch_bounds__(256) mlstm_scan_k(const E* __restrict__ q, int
   for (int tb = t0; tb < t1; tb += TC) {
     const int nt = min(TC, t1 - tb);
     __syncthreads();
-    for (int i = threadIdx.x; i < nt * DP; i += blockDim.x) {
-      const int tt = i / DP, c = i - tt * DP;
-      qs[i] = c < d ? ldf(q + (int64_t)(tb + tt) * q_ld + h * d + c) * qscale : 0.f;
-      ks[i] = c < d ? ldf(k + (int64_t)(tb + tt) * k_ld + h * d + c) : 0.f;
-    }
-    for (int i = threadIdx.x; i < nt * 64; i += blockDim.x) {
-      const int tt = i >> 6, col = blockIdx.z * 64 + (i & 63);
-      vs[i] = col < dv ? ldf(v + (int64_t)(tb + tt) * v_ld + h * dv + col) : 0.f;
+    if (vec) {
+      // 4-element chunks; a thread's loads are all issued before the first store
+      const int c4n = DP >> 2, n4 = nt * c4n;
+      float qv[4][4], kv[4][4];
+      int at[4];
+#pragma unroll
+      for (int u = 0; u < 4; u++) {
+        const int i = threadIdx.x + u * blockDim.x;
+        at[u] = -1;
+        if (i < n4) {
+          const int tt = i / c4n, c = (i - tt * c4n) * 4;
+          at[u] = tt * DP + c;
+          if (c < d) {
+            Ld4<E>::get(q + (int64_t)(tb + tt) * q_ld + h * d + c, qv[u]);
+            Ld4<E>::get(k + (int64_t)(tb + tt) * k_ld + h * d + c, kv[u]);
+          } else {
+#pragma unroll
+            for (int e = 0; e < 4; e++) qv[u][e] = kv[u][e] = 0.f;
+          }
+        }
+      }
+      float vv[4];
+      const int vi = threadIdx.x;                                     // 16 tokens x 16 chunks = 256 chunks at most
+      const int vt = vi >> 4, vc = blockIdx.z * 64 + (vi & 15) * 4;
+      const bool vok = vi < nt * 16;
+      if (vok) {
+        if (vc < dv) Ld4<E>::get(v + (int64_t)(tb + vt) * v_ld + h * dv + vc, vv);
+        else vv[0] = vv[1] = vv[2] = vv[3] = 0.f;
+      }
+#pragma unroll
+      for (int u = 0; u < 4; u++)
+        if (at[u] >= 0) {
+#pragma unroll
+          for (int e = 0; e < 4; e++) {
+            qs[at[u] + e] = qv[u][e] * qscale;
+            ks[at[u] + e] = kv[u][e];
+          }
+        }
+      if (blockDim.x < 256) {                                          // fewer threads than value chunks
+        for (int i = threadIdx.x; i < nt * 64; i += blockDim.x) {
+          const int tt = i >> 6, col = blockIdx.z * 64 + (i & 63);
+          vs[i] = col < dv ? ldf(v + (int64_t)(tb + tt) * v_ld + h * dv + col) : 0.f;
+        }
+      } else if (vok) {
+#pragma unroll
+        for (int e = 0; e < 4; e++) vs[vt * 64 + (vi & 15) * 4 + e] = vv[e];
+      }
+    } else {
+      for (int i = threadIdx.x; i < nt * DP; i += blockDim.x) {
+        const int tt = i / DP, c = i - tt * DP;
+        qs[i] = c < d ? ldf(q + (int64_t)(tb + tt) * q_ld + h * d + c) * qscale : 0.f;
+        ks[i] = c < d ? ldf(k + (int64_t)(tb + tt) * k_ld + h * d + c) : 0.f;
+      }
+      for (int i = threadIdx.x; i < nt * 64; i += blockDim.x) {
+        const int tt = i >> 6, col = blockIdx.z * 64 + (i & 63);
+        vs[i] = col < dv ? ldf(v + (int64_t)(tb + tt) * v_ld + h * dv + col) : 0.f;
+      }
     }
     for (int tt = threadIdx.x; tt < nt; tt += blockDim.x) {
       const float iz = (ldf(ipre + (int64_t)(tb + tt) * i_ld + h) + ib[h]) / cap;
@@ -612,7 +713,8 @@ static int pad_row(int D) {
 int latent_attention_plan(bool bf16, int H, int r, int dr, int* kt, int* nw, int* hbo) {
   const int esz = bf16 ? 2 : 4, D = r + dr;
   const int DP = pad_row(D), D4 = (D + 3) & ~3;
-  static const int opts[][2] = {{64, 4}, {64, 2}, {32, 4}, {32, 2}, {64, 1}, {16, 4}, {32, 1}, {16, 2}, {16, 1}};
+  // (keys per tile, waves): more waves first -- lanes are never idle whatever the tile size
+  static const int opts[][2] = {{64, 4}, {32, 4}, {16, 4}, {64, 2}, {32, 2}, {16, 2}, {64, 1}, {32, 1}, {16, 1}};
   // 16 heads per workgroup only while the f32 accumulators (heads x latent columns per lane) stay in registers
   for (int hb = (H > 8 && r <= 128) ? 16 : 8; hb >= 8; hb -= 8) {
     const size_t qbytes = ((size_t)hb * D4 * esz + 15) & ~(size_t)15;
@@ -695,10 +797,15 @@ void mlstm_scan(bool bf16, const void* q, int64_t q_ld, const void* k, int64_t k
   const int TC = 16;                       // tokens staged per chunk (52 KB of LDS at d = 256)
   const size_t lds = ((size_t)2 * TC * DP + (size_t)TC * 64 + (size_t)NWV * TC * 64 + 5 * (size_t)TC) * 4;
   dim3 grid(B, H, (dv + 63) / 64), block(64 * NWV);
+  // aligned 4-element loads: sizes, row strides and base addresses all multiples of 4 elements; the
+  // chunked staging covers 4 x 256 (q, k) chunks per 16 tokens
+  const size_t a4 = bf16 ? 8 : 16;
+  const bool vec = ((d | dv | q_ld | k_ld | v_ld) & 3) == 0 && (uintptr_t)q % a4 == 0 && (uintptr_t)k % a4 == 0 &&
+                   (uintptr_t)v % a4 == 0 && TC * (DP >> 2) <= 4 * 64 * NWV;
 #define SM_SCAN(DSV)                                                                                                  \
   SM_DISPATCH(bf16, hipLaunchKernelGGL((mlstm_scan_k<E, DSV>), grid, block, lds, st, (const E*)q, q_ld, (const E*)k,   \
                                        k_ld, (const E*)v, v_ld, (const E*)ipre, i_ld, (const E*)fpre, f_ld, ib, fb,    \
-                                       cap, S, n, m, cu, slots, pos, out, H, d, dv, TC))
+                                       cap, S, n, m, cu, slots, pos, out, H, d, dv, TC, vec))
   if (DS == 8) { SM_SCAN(8); }
   else if (DS == 16) { SM_SCAN(16); }
   else if (DS == 32) { SM_SCAN(32); }

@@ -122,6 +122,9 @@ class LLMEngine:
         self.metrics = EngineMetrics()
         self.use_graph = use_graph and not self.ragged and model.device.type == "cuda" and \
             ops.native_gpu(self.cache.k[0])
+        # ragged models: steps in which every sequence brings one token (pure
+        # decode) replay a hipGraph per (batch, table width) bucket
+        self.use_graph_ragged = bool(use_graph) and self.ragged and model.device.type == "cuda"
         self._graphs: Dict[tuple, dict] = {}
         # every captured (batch, width) bucket allocates from ONE private pool,
         # and only buckets whose forward is capture-safe are captured (MoE
@@ -396,6 +399,8 @@ class LLMEngine:
         entry order and marks the tokens as cached."""
         if not self.ragged:
             raise RuntimeError("run_batch: this model's forward takes uniform batches only")
+        if self.use_graph_ragged and all(len(e[1]) == 1 for e in entries):
+            return self._run_decode_graph(entries)
         m, dev, bs = self.model, self.model.device, self.block_size
         ids, pos, slots, seq_of, prev, lidx = [], [], [], [], [], []
         cu, ctx, qn, rows, sslots = [0], [], [], [], []
@@ -435,6 +440,77 @@ class LLMEngine:
             self.sched.advance(rid, len(toks))
             self._last_tok[rid] = int(toks[-1])
         return logits
+
+    def _capture_ragged(self, Bb: int, Wb: int) -> dict:
+        """hipGraph of one decode forward of a ragged model for Bb sequences
+        (padded rows: position 0 of the scratch block / scratch state slot)
+        with block tables Wb wide; slots and key counts are derived on the
+        device, so a replay needs ids, previous ids, positions, tables, slots."""
+        m, bs, dev = self.model, self.block_size, self.model.device
+        g = {"ids": torch.zeros(Bb, dtype=torch.long, device=dev),
+             "prev": torch.full((Bb,), -1, dtype=torch.long, device=dev),
+             "pos": torch.zeros(Bb, dtype=torch.long, device=dev),
+             "bt": torch.full((Bb, Wb), self._scratch, dtype=torch.int32, device=dev),
+             "ss": torch.full((Bb,), self.cache.num_slots, dtype=torch.int32, device=dev),
+             "cu": torch.arange(Bb + 1, dtype=torch.int32, device=dev),
+             "seq_of": torch.arange(Bb, dtype=torch.int32, device=dev)}
+        m.ensure_rope_cache(Wb * bs + 1)
+
+        def body():
+            pos, bt = g["pos"], g["bt"]
+            blk = torch.gather(bt, 1, (pos // bs).unsqueeze(1)).squeeze(1).long()
+            slots = blk * bs + pos % bs
+            meta = AttnMeta(Bb, 1, bt, (pos + 1).to(torch.int32), nsplit_for(Wb * bs), [Wb * bs] * Bb, cu_q=g["cu"],
+                            q_lens_host=[1] * Bb, seq_of=g["seq_of"], state_slots=g["ss"], prev_ids=g["prev"])
+            return m.forward_tokens(g["ids"], pos, slots, meta, self.cache)
+
+        s = torch.cuda.Stream()
+        s.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(s):            # warm-up: writes only the scratch block and the scratch slot
+            body()
+        torch.cuda.current_stream().wait_stream(s)
+        g["graph"] = torch.cuda.CUDAGraph()
+        if self._graph_pool is None:
+            self._graph_pool = torch.cuda.graph_pool_handle()
+        with torch.cuda.graph(g["graph"], pool=self._graph_pool):
+            g["logits"] = body()
+        self._graphs[("ragged", Bb, Wb)] = g
+        return g
+
+    def _run_decode_graph(self, entries) -> torch.Tensor:
+        B, bs = len(entries), self.block_size
+        rows, ids, pos, prev, ss, want = [], [], [], [], [], []
+        for i, (rid, toks, w) in enumerate(entries):
+            start = int(self.sched.cached(rid))
+            blocks = list(self.sched.blocks(rid))
+            if start + 1 > len(blocks) * bs:
+                raise RuntimeError(f"run_batch: sequence {rid} has no blocks for {start + 1} tokens")
+            rows.append(blocks)
+            ids.append(int(toks[0]))
+            pos.append(start)
+            prev.append(self._last_tok.get(rid, -1) if start > 0 else -1)
+            ss.append(max(int(self.sched.slot(rid)), 0))
+            want += [i] * len(w)
+        Bb = self._bucket(B)
+        Wb = self._bucket(max(len(x) for x in rows), 4)
+        g = self._graphs.get(("ragged", Bb, Wb)) or self._capture_ragged(Bb, Wb)
+        bt = torch.full((Bb, Wb), self._scratch, dtype=torch.int32)
+        for i, x in enumerate(rows):
+            bt[i, :len(x)] = torch.tensor(x, dtype=torch.int32)
+        pad = Bb - B
+        g["bt"].copy_(bt, non_blocking=True)
+        g["ids"].copy_(torch.tensor(ids + [0] * pad), non_blocking=True)
+        g["pos"].copy_(torch.tensor(pos + [0] * pad), non_blocking=True)
+        g["prev"].copy_(torch.tensor(prev + [-1] * pad), non_blocking=True)
+        g["ss"].copy_(torch.tensor(ss + [self.cache.num_slots] * pad, dtype=torch.int32), non_blocking=True)
+        g["graph"].replay()
+        for rid, toks, _ in entries:
+            self.sched.advance(rid, 1)
+            self._last_tok[rid] = int(toks[0])
+        lg = g["logits"]
+        if want == list(range(B)):
+            return lg[:B].clone()
+        return lg.index_select(0, torch.tensor(want, dtype=torch.long, device=lg.device))
 
     def open_stream(self) -> int:
         """Admit a sequence whose tokens are fed from outside with

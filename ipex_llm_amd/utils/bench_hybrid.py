@@ -55,7 +55,7 @@ def bench_hybrid(sz: dict, dev, prompt_len: int, batch: int, steps: int, warmup:
     total = prompt_len + warmup + steps + 8
     nblk = batch * (-(-total // 64))
     eng = LLMEngine(model, max_batch=batch, block_size=64, num_blocks=nblk, max_model_len=total,
-                    max_prefill_tokens=1 << 30, use_graph=False, enable_prefix_caching=False)
+                    max_prefill_tokens=1 << 30, use_graph=True, enable_prefix_caching=False)
     g = torch.Generator().manual_seed(0)
     prompts = [torch.randint(0, spec.vocab_size, (prompt_len,), generator=g).tolist() for _ in range(batch)]
     # prefill: one request, whole prompt, (warm-up run first)

@@ -379,6 +379,32 @@ def test_generation_survives_preemption(dev):
     assert eng.stats["preemptions"] >= 1
 
 
+@pytest.mark.gpu
+def test_decode_graph_replays_equal_eager():
+    """pure-decode steps replayed from a captured graph (padded batch bucket,
+    scratch block and slot for the padding rows), with eager prefill steps and
+    synchronisations between the replays: every replay equals the eager step"""
+    if not torch.cuda.is_available():
+        pytest.skip("no GPU")
+    from ipex_llm_amd.serving.engine import LLMEngine
+    dev = torch.device("cuda")
+    cfg = std_cfg()
+    W = O.random_weights(cfg, 24)
+    prompts = {"a": O.random_tokens(cfg, 90, 1), "b": O.random_tokens(cfg, 40, 2), "c": O.random_tokens(cfg, 75, 3)}
+    schedule = [[("a", 60), ("b", 20)], [("a", 1), ("b", 1)], [("a", 1), ("b", 1), ("c", 70)]] + \
+        [[("a", 1), ("b", 1), ("c", 1)]] * 5 + [[("a", 23), ("b", 1)]] + [[("b", 1)]] * 12
+    got = {}
+    for graph in (False, True):
+        eng = LLMEngine(build(cfg, W, dev, torch.float32), max_batch=4, block_size=64, num_blocks=12,
+                        max_model_len=512, max_prefill_tokens=1 << 30, use_graph=graph, enable_prefix_caching=False)
+        got[graph] = replay(eng, prompts, schedule)
+        assert bool(eng._graphs) == graph
+    for name, toks in prompts.items():
+        n = got[True][name].shape[0]
+        assert rel_err(got[True][name], got[False][name]) < 1e-4, name
+        assert rel_err(got[True][name], O.forward(cfg, W, toks)[:n]) < TOL[torch.float32], name
+
+
 # ------------------------------------------------------------------ checkpoint reader, registry, trace replay
 def write_checkpoint(path, cfg, W):
     from safetensors.torch import save_file
