@@ -16,6 +16,7 @@
 #include "seqmix.h"
 
 #include <math.h>
+#include <stdlib.h>
 
 namespace illm {
 namespace sm {
@@ -386,6 +387,206 @@ __global__ void __launch_bounds__(256) latent_attn_k(const E* __restrict__ q_lat
   }
 }
 
+// bf16 variant with the score products on the matrix cores: S^T = K Q^T as
+// 16x16x32 MFMAs (A = 16 key rows of the LDS tile, B = the head rows of the
+// staged query, both bf16 as stored; f32 accumulation), which leaves
+// (key = 4 g + i, head = lane & 15) in registers.  Softmax runs there in f32;
+// the f32 weights and each head's rescale factor go through LDS to the
+// weighted sum, which stays on the vector unit in f32 (weights are not
+// rounded).  Tiles are 16 keys; rows are padded to round_up(D, 32) + 8
+// elements (zero filled), so fragment reads are aligned and conflict-free.
+typedef __bf16 sm_bf16x8 __attribute__((ext_vector_type(8)));
+typedef float sm_f32x4 __attribute__((ext_vector_type(4)));
+
+template <int RC, int HB>
+__global__ void __launch_bounds__(256) latent_attn_mfma_k(const __bf16* __restrict__ q_lat, const __bf16* __restrict__ q_rot,
+                                                         int64_t qr_st, int64_t qr_sh, const __bf16* __restrict__ rows,
+                                                         int bs, const int32_t* __restrict__ bt, int bt_w,
+                                                         const int32_t* __restrict__ seq_of,
+                                                         const int64_t* __restrict__ pos, float scale,
+                                                         const __bf16* __restrict__ gate, int64_t g_st,
+                                                         __bf16* __restrict__ out, float* __restrict__ part, int H, int r,
+                                                         int dr, int DP) {
+  typedef __bf16 E;
+  constexpr int KT = 16;
+  extern __shared__ __align__(16) unsigned char smem[];
+  const int D = r + dr, KS = (D + 31) >> 5;                        // 32-wide product steps
+  const int nsplit = gridDim.z, zs = blockIdx.z;
+  const int t = blockIdx.x, h0 = blockIdx.y * HB;
+  const int nh = min(HB, H - h0);
+  const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6, NW = blockDim.x >> 6;
+  const int r16 = lane & 15, g = lane >> 4;
+  E* qs = (E*)smem;                                                // [16][DP], zero padded rows and columns
+  const size_t q_bytes = (size_t)16 * DP * sizeof(E);
+  const size_t wave_bytes = ((size_t)KT * DP * sizeof(E) + (size_t)HB * KT * sizeof(float) + 16 * sizeof(float) + 15) & ~(size_t)15;
+  unsigned char* wbase = smem + q_bytes + wv * wave_bytes;
+  E* kt = (E*)wbase;                                               // [KT][DP]
+  float* pb = (float*)(wbase + (size_t)KT * DP * sizeof(E));       // [HB][KT] weights
+  float* al = pb + HB * KT;                                        // [16] rescale factor per head
+  for (int i = threadIdx.x; i < 16 * DP; i += blockDim.x) stf(qs + i, 0.f);
+  for (int i = lane; i < KT * DP; i += 64) stf(kt + i, 0.f);
+  __syncthreads();
+  typedef uint2 C4;
+  if ((((int64_t)r | dr | qr_st | qr_sh) & 3) == 0 && ((uintptr_t)q_rot % sizeof(C4)) == 0) {
+#pragma unroll
+    for (int h = 0; h < HB; h++) {
+      if (h < nh) {
+        C4* dst = (C4*)(qs + h * DP);
+        const C4* a = (const C4*)(q_lat + ((int64_t)t * H + h0 + h) * r);
+        const C4* b = (const C4*)(q_rot + (int64_t)t * qr_st + (int64_t)(h0 + h) * qr_sh);
+        for (int i = threadIdx.x; i < (r >> 2); i += blockDim.x) dst[i] = a[i];
+        for (int i = threadIdx.x; i < (dr >> 2); i += blockDim.x) dst[(r >> 2) + i] = b[i];
+      }
+    }
+  } else {
+    for (int i = threadIdx.x; i < nh * D; i += blockDim.x) {
+      const int h = i / D, c = i - h * D;
+      qs[h * DP + c] = c < r ? q_lat[((int64_t)t * H + h0 + h) * r + c]
+                             : q_rot[(int64_t)t * qr_st + (int64_t)(h0 + h) * qr_sh + (c - r)];
+    }
+  }
+  __syncthreads();
+  const int64_t p = pos[t];
+  const int32_t* tab = bt + (int64_t)seq_of[t] * bt_w;
+  const int ntiles = (int)(p / KT) + 1;
+  float m_r = -INFINITY, l_r = 0.f;                                // of head r16 (the same in its four lanes)
+  float o[HB][RC];
+#pragma unroll
+  for (int h = 0; h < HB; h++)
+#pragma unroll
+    for (int c = 0; c < RC; c++) o[h][c] = 0.f;
+  for (int ti = zs * NW + wv; ti < ntiles; ti += NW * nsplit) {
+    const int64_t k0 = (int64_t)ti * KT;
+    const int nvalid = (int)min((int64_t)KT, p - k0 + 1);
+    const int64_t row0 = (int64_t)tab[k0 / bs] * bs + (k0 % bs);
+    const E* src = rows + row0 * D;
+    if ((D & 3) == 0) {
+      const C4* s4 = (const C4*)src;
+      const int n4 = nvalid * (D >> 2);
+      int j = 0, c = lane * 4;
+      while (c >= D) { c -= D; j++; }
+      for (int i = lane; i < n4; i += 64 * 4) {
+        C4 v[4];
+        int jj[4], cc[4];
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+          jj[u] = j;
+          cc[u] = c;
+          if (i + 64 * u < n4) v[u] = s4[i + 64 * u];
+          c += 256;
+          while (c >= D) { c -= D; j++; }
+        }
+#pragma unroll
+        for (int u = 0; u < 4; u++)
+          if (i + 64 * u < n4) *(C4*)(kt + jj[u] * DP + cc[u]) = v[u];
+      }
+    } else {
+      for (int i = lane; i < nvalid * D; i += 64) {
+        const int j = i / D, c = i - j * D;
+        kt[j * DP + c] = src[i];
+      }
+    }
+    wave_sync();
+    sm_f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+    const E* ka = kt + r16 * DP + 8 * g;
+    const E* qb = qs + r16 * DP + 8 * g;
+    for (int ks = 0; ks < KS; ks++) {
+      const sm_bf16x8 a = *(const sm_bf16x8*)(ka + 32 * ks);
+      const sm_bf16x8 b = *(const sm_bf16x8*)(qb + 32 * ks);
+      acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc, 0, 0, 0);
+    }
+    // lane: keys 4 g + i (i = 0..3) of head r16
+    float sv[4], mloc = -INFINITY;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      sv[i] = (4 * g + i) < nvalid ? acc[i] * scale : -INFINITY;
+      mloc = fmaxf(mloc, sv[i]);
+    }
+    mloc = fmaxf(mloc, __shfl_xor(mloc, 16, 64));
+    mloc = fmaxf(mloc, __shfl_xor(mloc, 32, 64));
+    const float mn = fmaxf(m_r, mloc);
+    const float alpha = m_r == -INFINITY ? 0.f : expf(m_r - mn);
+    float pv[4], lsum = 0.f;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      pv[i] = sv[i] == -INFINITY ? 0.f : expf(sv[i] - mn);
+      lsum += pv[i];
+    }
+    lsum += __shfl_xor(lsum, 16, 64);
+    lsum += __shfl_xor(lsum, 32, 64);
+    l_r = l_r * alpha + lsum;
+    m_r = mn;
+    if (r16 < HB) {
+      *(float4*)(pb + r16 * KT + 4 * g) = make_float4(pv[0], pv[1], pv[2], pv[3]);
+      if (g == 0) al[r16] = alpha;
+    }
+    wave_sync();
+#pragma unroll
+    for (int h = 0; h < HB; h++) {
+      const float a = al[h];
+#pragma unroll
+      for (int c = 0; c < RC; c++) o[h][c] *= a;
+    }
+    const int nv4 = (nvalid + 3) & ~3;
+    for (int j = 0; j < nv4; j += 4) {
+      float kv[4][RC];
+#pragma unroll
+      for (int jj = 0; jj < 4; jj++)
+#pragma unroll
+        for (int c = 0; c < RC; c++) {
+          const int col = lane + 64 * c;
+          kv[jj][c] = col < r ? ldf(kt + (j + jj) * DP + col) : 0.f;
+        }
+#pragma unroll
+      for (int h = 0; h < HB; h++) {
+        const float4 w4 = *(const float4*)(pb + h * KT + j);
+#pragma unroll
+        for (int c = 0; c < RC; c++)
+          o[h][c] = fmaf(w4.x, kv[0][c], fmaf(w4.y, kv[1][c], fmaf(w4.z, kv[2][c], fmaf(w4.w, kv[3][c], o[h][c]))));
+      }
+    }
+    wave_sync();
+  }
+  __syncthreads();
+  const int MS = HB * (r + 2);
+  float* mg = (float*)smem + (size_t)wv * MS;
+#pragma unroll
+  for (int h = 0; h < HB; h++)
+#pragma unroll
+    for (int c = 0; c < RC; c++) {
+      const int col = lane + 64 * c;
+      if (col < r) mg[h * (r + 2) + col] = o[h][c];
+    }
+  if (g == 0 && r16 < HB) {
+    mg[r16 * (r + 2) + r] = m_r;
+    mg[r16 * (r + 2) + r + 1] = l_r;
+  }
+  __syncthreads();
+  const float* m0 = (const float*)smem;
+  for (int i = threadIdx.x; i < nh * (r + 2); i += blockDim.x) {
+    const int h = i / (r + 2), c = i - h * (r + 2);
+    float M = -INFINITY;
+    for (int w = 0; w < NW; w++) M = fmaxf(M, m0[(size_t)w * MS + h * (r + 2) + r]);
+    float L = 0.f, O = 0.f;
+    for (int w = 0; w < NW; w++) {
+      const float* gp = m0 + (size_t)w * MS + h * (r + 2);
+      const float mw = gp[r];
+      const float f = mw == -INFINITY ? 0.f : expf(mw - M);
+      L += gp[r + 1] * f;
+      if (c < r) O += gp[c] * f;
+    }
+    if (nsplit > 1) {
+      float* pp = part + (((int64_t)t * H + h0 + h) * nsplit + zs) * (r + 2);
+      pp[c] = c < r ? O : (c == r ? M : L);
+    } else if (c < r) {
+      float v = O / L;
+      if (gate) v *= 1.0f / (1.0f + expf(-ldf(gate + (int64_t)t * g_st + h0 + h)));
+      stf(out + ((int64_t)t * H + h0 + h) * r + c, v);
+    }
+  }
+}
+
+
 // merge of the key splits: part [T, H, nsplit, r + 2] -> out [T, H, r]
 template <typename E>
 __global__ void __launch_bounds__(128) latent_attn_combine_k(const float* __restrict__ part, const E* __restrict__ gate,
@@ -732,9 +933,34 @@ int latent_attention_plan(bool bf16, int H, int r, int dr, int* kt, int* nw, int
   return -1;
 }
 
+// the bf16 MFMA variant: 16-key tiles, rows of round_up(D, 32) + 8 elements
+static int mfma_row(int D) { return ((D + 31) & ~31) + 8; }
+static int latent_attention_plan_mfma(int H, int r, int dr, int* nw, int* hbo) {
+  const int DP = mfma_row(r + dr);
+  for (int hb = (H > 8 && r <= 128) ? 16 : 8; hb >= 8; hb -= 8) {
+    const size_t qbytes = (size_t)16 * DP * 2;
+    const size_t wave = ((size_t)16 * DP * 2 + (size_t)hb * 16 * 4 + 16 * 4 + 15) & ~(size_t)15;
+    for (int w = 4; w >= 1; w--) {
+      const size_t total = qbytes + wave * w;
+      if (total <= 64 * 1024 && (size_t)w * hb * (r + 2) * 4 <= total) {
+        *nw = w;
+        *hbo = hb;
+        return (int)total;
+      }
+    }
+  }
+  return -1;
+}
+
+static const bool kUseMfma = []() {
+  const char* e = getenv("ILLM_LATENT_MFMA");
+  return !(e && e[0] == '0');
+}();
+
 int latent_attention_splits(bool bf16, int T, int H, int r, int dr, int max_ctx) {
   int KT = 0, NW = 0, hb = 8;
-  if (latent_attention_plan(bf16, H, r, dr, &KT, &NW, &hb) < 0) return 1;
+  if (bf16 && kUseMfma && latent_attention_plan_mfma(H, r, dr, &NW, &hb) > 0) KT = 16;
+  else if (latent_attention_plan(bf16, H, r, dr, &KT, &NW, &hb) < 0) return 1;
   const int64_t blocks = (int64_t)T * ((H + hb - 1) / hb);
   const int tiles = (max_ctx + KT - 1) / KT;
   int ns = (int)((1024 + blocks - 1) / blocks);            // ~4 workgroups per CU
@@ -747,11 +973,36 @@ void latent_attention(bool bf16, const void* q_lat, const void* q_rot, int64_t q
                       float scale, const void* gate, int64_t g_st, void* out, float* part, int nsplit, int T, int H,
                       int r, int dr, hipStream_t st) {
   if (T <= 0) return;
+  const int rc = (r + 63) / 64;
   int KT = 0, NW = 0, hb = 8;
+  if (bf16 && kUseMfma) {
+    const int lds = latent_attention_plan_mfma(H, r, dr, &NW, &hb);
+    if (lds > 0) {
+      const int DP = mfma_row(r + dr);
+      dim3 grid(T, (H + hb - 1) / hb, nsplit), block(64 * NW);
+#define SM_ATTN_M(RC, HBV)                                                                                            \
+  hipLaunchKernelGGL((latent_attn_mfma_k<RC, HBV>), grid, block, lds, st, (const __bf16*)q_lat, (const __bf16*)q_rot,  \
+                     qr_st, qr_sh, (const __bf16*)rows, bs, block_tables, bt_width, seq_of, pos, scale,                \
+                     (const __bf16*)gate, g_st, (__bf16*)out, part, H, r, dr, DP)
+      if (hb == 8) {
+        if (rc <= 1) { SM_ATTN_M(1, 8); }
+        else if (rc <= 2) { SM_ATTN_M(2, 8); }
+        else if (rc <= 4) { SM_ATTN_M(4, 8); }
+        else { SM_ATTN_M(8, 8); }
+      } else {
+        if (rc <= 1) { SM_ATTN_M(1, 16); }
+        else { SM_ATTN_M(2, 16); }
+      }
+#undef SM_ATTN_M
+      if (nsplit > 1)
+        hipLaunchKernelGGL(latent_attn_combine_k<__bf16>, dim3(T, H), dim3(128), 0, st, part, (const __bf16*)gate, g_st,
+                           (__bf16*)out, H, r, nsplit);
+      return;
+    }
+  }
   const int lds = latent_attention_plan(bf16, H, r, dr, &KT, &NW, &hb);
   if (lds < 0) return;                     // refused by the caller beforehand
   const int DP = pad_row(r + dr);
-  const int rc = (r + 63) / 64;
   dim3 grid(T, (H + hb - 1) / hb, nsplit), block(64 * NW);
 #define SM_ATTN(RC, HBV)                                                                                              \
   SM_DISPATCH(bf16, hipLaunchKernelGGL((latent_attn_k<E, RC, HBV>), grid, block, lds, st, (const E*)q_lat,             \
@@ -764,9 +1015,7 @@ void latent_attention(bool bf16, const void* q_lat, const void* q_rot, int64_t q
     else { SM_ATTN(8, 8); }
   } else {
     if (rc <= 1) { SM_ATTN(1, 16); }
-    else if (rc <= 2) { SM_ATTN(2, 16); }
-    else if (rc <= 4) { SM_ATTN(4, 16); }
-    else { SM_ATTN(8, 16); }
+    else { SM_ATTN(2, 16); }
   }
 #undef SM_ATTN
   if (nsplit > 1) {

@@ -212,6 +212,32 @@ def test_far_key_stands_out(dev, key_at):
                 assert (out[i, 1] - 3.0 * mark[:r].double()).abs().max() < 1e-3
 
 
+@pytest.mark.parametrize("H,r,dr", [(3, 20, 6), (16, 512, 64), (9, 72, 8), (16, 96, 32), (1, 4, 2)])
+def test_latent_attention_op_bf16(dev, H, r, dr):
+    """the 16-bit kernel variant (scores on the matrix cores, f32 softmax and
+    weighted sum) on a ragged batch: a short portion of one sequence beside
+    single tokens of two others, shuffled pages, gate on"""
+    from ipex_llm_amd.ops import seqmix as SM
+    g = torch.Generator().manual_seed(H * 1000 + r)
+    bs = 64
+    rows = (0.5 * torch.randn(12, bs, r + dr, generator=g)).to(torch.bfloat16)
+    bt = torch.tensor([[7, 2, 9, 0], [4, 11, 1, 0], [5, 3, 0, 0]], dtype=torch.int32)
+    ctx, qn = [200, 130, 70], [9, 1, 1]
+    pos = torch.tensor(list(range(191, 200)) + [129, 69])
+    seq = torch.tensor([0] * 9 + [1, 2], dtype=torch.int32)
+    T = 11
+    q = (torch.randn(T, H, r + dr, generator=g) * 0.7).to(torch.bfloat16)
+    gate = torch.randn(T, H, generator=g).to(torch.bfloat16)
+    out = SM.latent_attention(q[..., :r].contiguous().to(dev), q[..., r:].to(dev), rows.to(dev), bt.to(dev), seq.to(dev),
+                              pos.to(dev), 0.11, gate.to(dev), qn, ctx, torch.bfloat16).float().cpu().double()
+    for i in range(T):
+        b = int(seq[i])
+        dense = torch.cat([rows[int(x)] for x in bt[b]])[:int(pos[i]) + 1].double()
+        sc = (dense @ q[i].double().T) * 0.11
+        want = (torch.softmax(sc, 0).T @ dense[:, :r]) * torch.sigmoid(gate[i].double())[:, None]
+        assert (out[i] - want).abs().max() < 6e-3 * max(1.0, float(want.abs().max())), i
+
+
 @pytest.mark.parametrize("qpos", [62, 63, 64, 65, 127, 128, 129])
 def test_causal_edge_at_page_borders(dev, qpos):
     """a towering key one position AFTER the query must not be seen; the same key AT the query must"""
