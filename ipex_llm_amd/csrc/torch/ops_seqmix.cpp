@@ -106,6 +106,14 @@ void sm_latent_kv_store(const Tensor& dkv, const Tensor& norm_w, double eps, int
                             slots.data_ptr<int64_t>(), rows.data_ptr(), rows.size(0) * rows.size(1), (int)T, stream());
 }
 
+// dynamic LDS the flash kernel would take for these sizes; -1: they do not fit (callers then take the
+// library-product path, which has no size limits)
+int64_t sm_latent_attention_fits(bool bf16, int64_t H, int64_t r, int64_t dr) {
+  if (r < 1 || r > 512) return -1;
+  int kt = 0, nw = 0, hb = 0;
+  return illm::sm::latent_attention_plan(bf16, (int)H, (int)r, (int)dr, &kt, &nw, &hb);
+}
+
 Tensor sm_latent_attention(const Tensor& q_lat, const Tensor& q_rot, const Tensor& rows, const Tensor& block_tables,
                            const Tensor& seq_of, const Tensor& pos, double scale, const c10::optional<Tensor>& gate,
                            int64_t max_ctx, bool act_f32) {
@@ -250,11 +258,16 @@ TORCH_LIBRARY_FRAGMENT(ipex_llm_amd, m) {
         "Tensor(a!) rows) -> ()");
   m.def("sm_latent_attention(Tensor q_lat, Tensor q_rot, Tensor rows, Tensor block_tables, Tensor seq_of, Tensor pos, "
         "float scale, Tensor? gate, int max_ctx, bool act_f32) -> Tensor");
+  m.def("sm_latent_attention_fits(bool bf16, int H, int r, int dr) -> int");
   m.def("sm_mlstm_scan(Tensor q, Tensor k, Tensor v, Tensor ipre, Tensor fpre, Tensor ib, Tensor fb, float cap, "
         "Tensor(a!) S, Tensor(b!) n, Tensor(c!) m, Tensor cu, Tensor slots, Tensor pos, int max_q) -> Tensor");
   m.def("sm_causal_softmax(Tensor(a!) scores, Tensor pos, int H, float scale, bool act_f32) -> (Tensor, Tensor)");
   m.def("sm_head_rms_gate(Tensor h, Tensor norm_w, Tensor gate, float eps, bool act_f32) -> Tensor");
   m.def("sm_glu_gelu(Tensor gu) -> Tensor");
+}
+
+TORCH_LIBRARY_IMPL(ipex_llm_amd, CompositeExplicitAutograd, m) {
+  m.impl("sm_latent_attention_fits", &sm_latent_attention_fits);
 }
 
 TORCH_LIBRARY_IMPL(ipex_llm_amd, CUDA, m) {

@@ -231,14 +231,16 @@ def _latent_attention_gemm(q_lat, q_rot, rows, table_row, pos, scale, L: int, n:
 def _latent_attention_gpu(q_lat, q_rot, rows, block_tables, seq_of, pos, scale, gate, q_lens, ctx_lens, out_dtype):
     T, H, r = q_lat.shape
     f32 = out_dtype == torch.float32
-    big = [b for b, n in enumerate(q_lens) if n >= GEMM_MIN_Q]
+    # sizes the flash kernel cannot hold in LDS / registers: every portion takes the library-product path
+    min_q = GEMM_MIN_Q if _ops().sm_latent_attention_fits(not f32, H, r, q_rot.shape[-1]) > 0 else 1
+    big = [b for b, n in enumerate(q_lens) if n >= min_q]
     if not big:
         return _ops().sm_latent_attention(q_lat.contiguous(), q_rot, rows, block_tables, seq_of, pos, scale, gate,
                                           max(ctx_lens), f32)
     out = torch.empty(T, H, r, dtype=out_dtype, device=q_lat.device)
     small, small_ctx, t0 = [], 1, 0
     for b, (n, L) in enumerate(zip(q_lens, ctx_lens)):
-        if n >= GEMM_MIN_Q:
+        if n >= min_q:
             o = _latent_attention_gemm(q_lat[t0:t0 + n], q_rot[t0:t0 + n], rows, block_tables[b], pos[t0:t0 + n], scale,
                                        L, n)
             if gate is not None:
@@ -276,7 +278,7 @@ def mlstm_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, i_pre: torch.T
     Returns h f32 [T, H, dv]."""
     T, H, d = q.shape
     dv = v.shape[-1]
-    if native(q):
+    if native(q) and d <= 256:          # (larger key sizes: the token loop below, on the device)
         return _ops().sm_mlstm_scan(q, k, v, i_pre, f_pre, i_bias, f_bias, float(cap), state["S"], state["n"],
                                     state["m"], cu, state_slots, pos, max(q_lens))
     out = torch.empty(T, H, dv, dtype=torch.float32, device=q.device)

@@ -376,6 +376,32 @@ def test_other_sizes_and_orders(dev):
         assert rel_err(got, O.forward(cfg, W, toks)) < TOL[torch.float32]
 
 
+ODD = [
+    # sizes that are not multiples of 4 (no aligned chunks anywhere), partial rotation
+    ([O.attn_layer(heads=5, dim=6, rot_dim=6, vdim=10, kv_rank=13, dims=4, ff=20), O.mlstm_layer(heads=3, dim=5, vdim=7)], 36),
+    # > 16 heads, latent rank past 256, key size 256 in the recurrence
+    ([O.attn_layer(heads=20, dim=16, rot_dim=16, vdim=16, kv_rank=300, ff=0, scaling=YARN),
+      O.mlstm_layer(heads=2, dim=256, vdim=64, gate_cap=8.0, ff=32)], 64),
+    # past what the flash kernel and the register-resident scan hold: the paths without size limits
+    ([O.attn_layer(heads=2, dim=8, rot_dim=8, vdim=8, kv_rank=520, ff=0), O.mlstm_layer(heads=1, dim=260, vdim=8)], 32),
+    # 16 heads with a small latent, key size that pads to the next wave slice
+    ([O.mlstm_layer(heads=2, dim=100, vdim=36, ff=0), O.attn_layer(heads=16, dim=32, rot_dim=32, vdim=32, kv_rank=96, ff=40)], 48),
+]
+
+
+@pytest.mark.parametrize("case", range(len(ODD)))
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_odd_and_large_sizes(dev, case, dtype):
+    """a long portion (the library-product path of the attention on the GPU),
+    a short one, then single tokens -- in both number formats"""
+    layers, width = ODD[case]
+    cfg = O.config(layers, vocab=61, width=width, eps=1e-6, mult=0.7, buckets=17, mul_prev=3, mul_cur=11)
+    W = O.random_weights(cfg, 30 + case)
+    toks = O.random_tokens(cfg, 170, 30 + case)
+    got = replay(engine(cfg, W, dev, dtype), {"a": toks}, [[("a", 140)], [("a", 20)]] + [[("a", 1)]] * 10)["a"]
+    assert rel_err(got, O.forward(cfg, W, toks)) < TOL[dtype]
+
+
 # ------------------------------------------------------------------ generation through the scheduler
 def test_greedy_generation_scheduler(dev):
     """LLMEngine.generate: C++ scheduler, chunked prompts (7 tokens a step in
