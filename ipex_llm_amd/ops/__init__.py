@@ -72,7 +72,11 @@ def require_seqmix():
             return torch.ops.ipex_llm_amd
         full = os.path.exists(_LIB_PATH)
     if full:
-        return require()
+        lib = require()
+        if not hasattr(lib, "sm_latent_attention"):
+            raise RuntimeError(f"{_LIB_PATH} predates the sequence-mixing kernels: rebuild it "
+                               "(python -m ipex_llm_amd._build)")
+        return lib
     with _lock:
         from .. import _build
         stale = _build.needs_build("seqmix")

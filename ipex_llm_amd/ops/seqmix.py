@@ -279,8 +279,7 @@ def mlstm_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, i_pre: torch.T
     T, H, d = q.shape
     dv = v.shape[-1]
     if native(q) and d <= 256:          # (larger key sizes: the token loop below, on the device)
-        return _ops().sm_mlstm_scan(q, k, v, i_pre, f_pre, i_bias, f_bias, float(cap), state["S"], state["n"],
-                                    state["m"], cu, state_slots, pos, max(q_lens))
+        return _mlstm_scan_gpu(q, k, v, i_pre, f_pre, i_bias, f_bias, float(cap), state, cu, state_slots, pos, q_lens)
     out = torch.empty(T, H, dv, dtype=torch.float32, device=q.device)
     ig = cap * torch.tanh((i_pre.float() + i_bias.float()) / cap)
     fg = F.logsigmoid(cap * torch.tanh((f_pre.float() + f_bias.float()) / cap))
@@ -308,6 +307,109 @@ def mlstm_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, i_pre: torch.T
             out[t] = torch.einsum("hdv,hd->hv", S, qf[t]) / den[:, None]
         state["S"][sl], state["n"][sl], state["m"][sl] = S, n, m
         t0 += nq
+    return out
+
+
+# Portions of at least MLSTM_CHUNK_MIN tokens take the chunk-parallel form on
+# the GPU: the recurrence is linear in the state, so within a chunk of C tokens
+#   m_t   = F_t + max(M, max_{s<=t}(i_s - F_s))            F: prefix sums of f in the chunk, M: m at its start
+#   num_t = e^{F_t + M - m_t} q_t^T S + sum_{s<=t} e^{F_t - F_s + i_s - m_t} (q_t . k_s) v_s
+# (and the same with n for the normaliser), every exponent <= 0.  The pairwise
+# part of all chunks and the chunk-end state increments K^T diag(w) V are
+# batched f32 products; only S_{c+1} = e^{..} S_c + U_c runs chunk after chunk.
+# Everything is f32; the token-sequential kernel takes what is left over.
+MLSTM_CHUNK = int(__import__("os").environ.get("ILLM_MLSTM_CHUNK", "128"))
+# None: by state size -- 512 tokens for large states (d x dv >= 64 K, where the sequential kernel's token
+# takes longest), 2048 otherwise (measured on MI355X: below these the one-launch kernel is faster)
+MLSTM_CHUNK_MIN = (lambda e: int(e) if e else None)(__import__("os").environ.get("ILLM_MLSTM_CHUNK_MIN"))
+
+
+def _chunk_min(d: int, dv: int) -> int:
+    if MLSTM_CHUNK_MIN is not None:
+        return max(MLSTM_CHUNK_MIN, MLSTM_CHUNK)
+    return max(MLSTM_CHUNK, 512 if d * dv >= 65536 else 2048)
+
+
+def mlstm_chunked(q, k, v, ig, fg, S0, n0, m0, C: int):
+    """q (already scaled), k [n, H, d], v [n, H, dv], log gates ig, fg [n, H],
+    all f32, n a multiple of C; S0 [H, d, dv], n0 [H, d], m0 [H].  Returns
+    h [n, H, dv] and the state after the last token."""
+    n, H, d = q.shape
+    dv = v.shape[-1]
+    NC = n // C
+    Q = q.view(NC, C, H, d).permute(2, 0, 1, 3)
+    K = k.view(NC, C, H, d).permute(2, 0, 1, 3)
+    V = v.view(NC, C, H, dv).permute(2, 0, 1, 3)
+    I = ig.view(NC, C, H).permute(2, 0, 1)
+    F_ = fg.view(NC, C, H).permute(2, 0, 1).cumsum(-1)                # [H, NC, C]
+    g = I - F_
+    G = g.cummax(-1).values
+    Ftot, Gtot = F_[..., -1], G[..., -1]                                # [H, NC]
+    # m at every chunk start: M_{c+1} = Ftot_c + max(M_c, Gtot_c) (scalars per head: on the host)
+    Fh, Gh = Ftot.cpu(), Gtot.cpu()
+    Ms = torch.empty(H, NC + 1, dtype=torch.float32)
+    Ms[:, 0] = m0.cpu()
+    for c in range(NC):
+        Ms[:, c + 1] = Fh[:, c] + torch.maximum(Ms[:, c], Gh[:, c])
+    Ms = Ms.to(q.device)
+    Mc, Mn = Ms[:, :-1], Ms[:, 1:]
+    m = F_ + torch.maximum(Mc[..., None], G)                            # [H, NC, C]
+    dec_in = torch.exp(F_ + Mc[..., None] - m)
+    vis = torch.ones(C, C, dtype=torch.bool, device=q.device).tril()
+    D = torch.exp(((F_ - m)[..., :, None] + g[..., None, :]).masked_fill(~vis, float("-inf")))
+    A = torch.matmul(Q, K.transpose(-1, -2)) * D                        # [H, NC, C, C]
+    w = torch.exp(Ftot[..., None] - F_ + I - Mn[..., None])             # weight of token s in the chunk-end state
+    U = torch.matmul(K.transpose(-1, -2), w[..., None] * V)             # [H, NC, d, dv]
+    un = torch.matmul(K.transpose(-1, -2), w[..., None]).squeeze(-1)    # [H, NC, d]
+    dec = torch.exp(Ftot + Mc - Mn)
+    S_all = torch.empty(H, NC + 1, d, dv, dtype=torch.float32, device=q.device)
+    n_all = torch.empty(H, NC + 1, d, dtype=torch.float32, device=q.device)
+    S_all[:, 0], n_all[:, 0] = S0, n0
+    for c in range(NC):
+        torch.addcmul(U[:, c], S_all[:, c], dec[:, c, None, None], out=S_all[:, c + 1])
+        torch.addcmul(un[:, c], n_all[:, c], dec[:, c, None], out=n_all[:, c + 1])
+    num = torch.matmul(A, V) + dec_in[..., None] * torch.matmul(Q, S_all[:, :-1])
+    nq = A.sum(-1) + dec_in * torch.matmul(Q, n_all[:, :-1, :, None]).squeeze(-1)
+    den = torch.maximum(nq.abs(), torch.exp(-m)) + 1e-6
+    h = (num / den[..., None]).permute(1, 2, 0, 3).reshape(n, H, dv)
+    return h, S_all[:, -1], n_all[:, -1], Ms[:, -1]
+
+
+def _mlstm_scan_gpu(q, k, v, i_pre, f_pre, i_bias, f_bias, cap, state, cu, state_slots, pos, q_lens):
+    T, H, d = q.shape
+    dv = v.shape[-1]
+    C = MLSTM_CHUNK
+    cmin = _chunk_min(d, dv)
+    if max(q_lens) < cmin:
+        return _ops().sm_mlstm_scan(q, k, v, i_pre, f_pre, i_bias, f_bias, cap, state["S"], state["n"], state["m"],
+                                    cu, state_slots, pos, max(q_lens))
+    out = torch.empty(T, H, dv, dtype=torch.float32, device=q.device)
+    slots = state_slots.tolist()
+    rest, rest_lens, rest_slots, t0 = [], [], [], 0              # what the sequential kernel takes afterwards
+    for b, nq in enumerate(q_lens):
+        nfull = (nq // C) * C if nq >= cmin else 0
+        if nfull:
+            sl, r = slots[b], slice(t0, t0 + nfull)
+            ig = cap * torch.tanh((i_pre[r].float() + i_bias) / cap)
+            fg = F.logsigmoid(cap * torch.tanh((f_pre[r].float() + f_bias) / cap))
+            fresh = int(pos[t0]) == 0
+            S0 = torch.zeros(H, d, dv, device=q.device) if fresh else state["S"][sl]
+            n0 = torch.zeros(H, d, device=q.device) if fresh else state["n"][sl]
+            m0 = torch.zeros(H, device=q.device) if fresh else state["m"][sl]
+            h, S1, n1, m1 = mlstm_chunked(q[r].float() * d ** -0.5, k[r].float(), v[r].float(), ig, fg, S0, n0, m0, C)
+            out[r] = h
+            state["S"][sl], state["n"][sl], state["m"][sl] = S1, n1, m1
+        if nq - nfull:
+            rest.append(torch.arange(t0 + nfull, t0 + nq, device=q.device))
+            rest_lens.append(nq - nfull)
+            rest_slots.append(slots[b])
+        t0 += nq
+    if rest:
+        idx = torch.cat(rest)
+        cu_r = torch.tensor([0] + list(__import__("itertools").accumulate(rest_lens)), dtype=torch.int32, device=q.device)
+        ss_r = torch.tensor(rest_slots, dtype=torch.int32, device=q.device)
+        out[idx] = _ops().sm_mlstm_scan(q[idx], k[idx], v[idx], i_pre[idx], f_pre[idx], i_bias, f_bias, cap, state["S"],
+                                        state["n"], state["m"], cu_r, ss_r, pos[idx].contiguous(), max(rest_lens))
     return out
 
 

@@ -127,6 +127,33 @@ def test_mlstm_alone(dev, layer):
     assert rel_err(got, O.forward(cfg, W, toks)) < TOL[torch.float32]
 
 
+@pytest.mark.parametrize("C", [4, 32])
+def test_mlstm_chunk_parallel_form(dev, C):
+    """the chunk-parallel form of the recurrence against the token loop, continuing from a non-zero state"""
+    from ipex_llm_amd.ops import seqmix as SM
+    g = torch.Generator().manual_seed(C)
+    n, H, d, dv = 96, 3, 10, 14
+    q, k = torch.randn(n, H, d, generator=g) * d ** -0.5, torch.randn(n, H, d, generator=g)
+    v = torch.randn(n, H, dv, generator=g)
+    ig = 3.0 * torch.tanh(torch.randn(n, H, generator=g) * 2)
+    fg = torch.nn.functional.logsigmoid(3.0 * torch.tanh(torch.randn(n, H, generator=g) * 2 + 1))
+    S0, n0, m0 = torch.randn(H, d, dv, generator=g), torch.randn(H, d, generator=g), torch.rand(H, generator=g) * 2
+    h, S1, n1, m1 = SM.mlstm_chunked(*(x.to(dev) for x in (q, k, v, ig, fg, S0, n0, m0)), C)
+    S, nn, m = S0.double(), n0.double(), m0.double()
+    want = torch.zeros(n, H, dv, dtype=torch.float64)
+    for t in range(n):
+        mn = torch.maximum(fg[t].double() + m, ig[t].double())
+        a, b = torch.exp(fg[t].double() + m - mn), torch.exp(ig[t].double() - mn)
+        S = a[:, None, None] * S + b[:, None, None] * k[t].double()[:, :, None] * v[t].double()[:, None, :]
+        nn = a[:, None] * nn + b[:, None] * k[t].double()
+        m = mn
+        den = torch.maximum((nn * q[t].double()).sum(-1).abs(), torch.exp(-m)) + 1e-6
+        want[t] = torch.einsum("hdv,hd->hv", S, q[t].double()) / den[:, None]
+    assert (h.cpu().double() - want).abs().max() < 2e-4 * max(1.0, float(want.abs().max()))
+    assert (S1.cpu().double() - S).abs().max() < 2e-4 * max(1.0, float(S.abs().max()))
+    assert (n1.cpu().double() - nn).abs().max() < 2e-4 and (m1.cpu().double() - m).abs().max() < 1e-5
+
+
 def test_mlstm_gates_saturate(dev):
     """large pre-activations: the cap bounds both gates, the running maximum keeps exp() finite"""
     cfg = O.config([O.mlstm_layer(heads=2, dim=8, vdim=8, gate_cap=6.0)], mult=1.0)
@@ -337,6 +364,21 @@ def test_pages_and_slots_used_again(dev):
     with pytest.raises(RuntimeError):                  # a third live request has no slot
         for _ in range(3):
             eng.open_stream()
+
+
+def test_long_portions_chunk_parallel(dev, monkeypatch):
+    """portions long enough for the chunk-parallel recurrence and the
+    library-product attention (on the GPU), cut so that both leave remainders,
+    beside a short request in the same steps"""
+    from ipex_llm_amd.ops import seqmix as SM
+    monkeypatch.setattr(SM, "MLSTM_CHUNK_MIN", 256)
+    cfg = std_cfg()
+    W = O.random_weights(cfg, 25)
+    prompts = {"a": O.random_tokens(cfg, 700, 25), "b": O.random_tokens(cfg, 9, 26)}
+    got = replay(engine(cfg, W, dev, num_blocks=16), prompts,
+                 [[("a", 300), ("b", 3)], [("a", 390), ("b", 1)], [("a", 10), ("b", 5)]])
+    for name, toks in prompts.items():
+        assert rel_err(got[name], O.forward(cfg, W, toks)) < TOL[torch.float32], name
 
 
 def test_long_decoding(dev):
