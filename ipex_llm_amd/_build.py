@@ -81,7 +81,7 @@ def _cmd(src: str, obj: str):
             # some of them (profiles/gemv5_xm_forms_r6.txt)
             if os.path.basename(src) == "gemv_int4_xm.hip":
                 extra = ["-fno-slp-vectorize"]
-        if os.path.basename(src) == "seqmix.hip":
+        if os.path.basename(src) == "seqmix.hip" or os.path.basename(src).startswith("blockmix_"):
             # f32-exact kernels: no packed-f32 instruction forms
             extra = ["-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
         return [HIPCC, f"--offload-arch={ARCH}", "-Wno-pass-failed", *extra, *common, "-c", src, "-o", obj]
@@ -96,7 +96,8 @@ def _cmd(src: str, obj: str):
 # partial libraries: the translation units one model kind needs, linked alone
 TARGETS = {
     # hybrid decoders: sequence-mixing kernels + their bindings + the serving scheduler
-    "seqmix": ["hip/seqmix.hip", "torch/ops_seqmix.cpp", "runtime/scheduler.cpp"],
+    "seqmix": ["hip/seqmix.hip", "hip/blockmix_elem.hip", "hip/blockmix_attn.hip", "hip/blockmix_moe.hip",
+               "torch/ops_seqmix.cpp", "torch/ops_blockmix.cpp", "runtime/scheduler.cpp"],
 }
 
 

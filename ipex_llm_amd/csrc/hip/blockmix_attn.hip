@@ -1,0 +1,468 @@
+// Grouped-query attention with mixed head scores over paged [keys | values]
+// rows (gfx950, wave64).
+//
+//   qk_norm_rope_store_k   per-head RMS norm + half-split rotary positions on
+//                          queries and keys, cache append of [normed rotated
+//                          keys | keys as projected]; queries leave in f32
+//   talk_attn_k            one workgroup per (query token, key split): all H
+//                          heads of the token together, because the scores of
+//                          all heads at a key are mixed by an [H, H] matrix
+//                          before the softmax.  Per key tile: scores (f32),
+//                          mixing, causal mask, online softmax, weighted sum
+//                          of the values (f32 accumulators in registers).
+//   talk_attn_combine_k    merge of the key splits + sigmoid output gate
+//   talk_softmax_k         the scale + mixing + mask + softmax step of the
+//                          library-product path of long portions
+//
+// Cache rows are bf16 or f32 (template E); queries, scores and weights are f32.
+#include "blockmix.h"
+
+#include <math.h>
+
+namespace illm {
+namespace bm {
+namespace {
+
+template <typename E> __device__ __forceinline__ float ldf(const E* p);
+template <> __device__ __forceinline__ float ldf<float>(const float* p) { return *p; }
+template <> __device__ __forceinline__ float ldf<__bf16>(const __bf16* p) { return (float)*p; }
+template <typename E> __device__ __forceinline__ void stf(E* p, float v);
+template <> __device__ __forceinline__ void stf<float>(float* p, float v) { *p = v; }
+template <> __device__ __forceinline__ void stf<__bf16>(__bf16* p, float v) { *p = (__bf16)v; }
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+  return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+  return v;
+}
+__device__ __forceinline__ void wave_sync() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+// ------------------------------------------------------------------ norm + rotary + cache append
+// one block per token, one wave per head in turn (query heads, then key heads); buf: 4 x d floats
+template <typename E>
+__global__ void __launch_bounds__(256) qk_norm_rope_store_k(const E* __restrict__ q, int64_t q_ld, const E* __restrict__ k,
+                                                           int64_t k_ld, const E* __restrict__ qn, const E* __restrict__ kn,
+                                                           float eps, const float* __restrict__ table, int max_pos,
+                                                           int dims, const int64_t* __restrict__ pos,
+                                                           const int64_t* __restrict__ slots, E* __restrict__ rows,
+                                                           int64_t num_rows, float* __restrict__ qo, int H, int G, int d) {
+  extern __shared__ float buf_all[];
+  const int64_t t = blockIdx.x;
+  const int wv = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  float* buf = buf_all + wv * d;
+  int64_t p = pos[t];
+  const bool in_table = p >= 0 && p < max_pos;
+  if (!in_table) p = 0;
+  const float* cs = table + p * dims;               // [dims / 2][2]
+  const int half = dims >> 1;
+  const int64_t slot = slots[t];
+  const bool store = slot >= 0 && slot < num_rows;
+  for (int hh = wv; hh < H + G; hh += 4) {
+    const bool isq = hh < H;
+    const E* src = isq ? q + t * q_ld + (int64_t)hh * d : k + t * k_ld + (int64_t)(hh - H) * d;
+    const E* nw = isq ? qn : kn;
+    float ss = 0.f;
+    for (int i = lane; i < d; i += 64) {
+      const float v = ldf(src + i);
+      ss += v * v;
+    }
+    const float rs = nw ? 1.0f / sqrtf(wave_sum(ss) / (float)d + eps) : 1.0f;
+    for (int i = lane; i < d; i += 64) buf[i] = ldf(src + i) * rs * (nw ? ldf(nw + i) : 1.0f);
+    wave_sync();
+    E* krow = store ? rows + slot * (int64_t)(2 * G * d) + (int64_t)(hh - H) * d : nullptr;
+    for (int i = lane; i < d; i += 64) {
+      float v = buf[i];
+      if (i < dims && in_table) {
+        const int j = i < half ? i : i - half;
+        const float c = cs[2 * j], s = cs[2 * j + 1];
+        v = i < half ? buf[i] * c - buf[i + half] * s : buf[i] * c + buf[i - half] * s;
+      }
+      if (isq) qo[(t * H + hh) * d + i] = v;
+      else if (krow) {
+        stf(krow + i, v);
+        krow[(int64_t)G * d + i] = src[i];
+      }
+    }
+    wave_sync();
+  }
+}
+
+// ------------------------------------------------------------------ flash kernel
+constexpr int kMaxItems = 4;        // (kv head, value column) items per thread: G d <= 1024
+
+template <typename E> struct Words;   // a 4-byte word of cache row
+template <> struct Words<float> {
+  static constexpr int per = 1;
+  static __device__ __forceinline__ void get(uint32_t w, float* v) { v[0] = __uint_as_float(w); }
+};
+template <> struct Words<__bf16> {
+  static constexpr int per = 2;
+  static __device__ __forceinline__ void get(uint32_t w, float* v) {
+    v[0] = __uint_as_float(w << 16);
+    v[1] = __uint_as_float(w & 0xffff0000u);
+  }
+};
+
+// LDS layout (floats unless noted): qs [H d] | tk [H H] | S [H (KT + 1)] | S2 [H (KT + 1)] | mrun lrun corr [3 H] |
+// red [JS H d] | tile (uint32 words) [KT pitch_w]
+template <typename E, int REP>
+__global__ void __launch_bounds__(256) talk_attn_k(const float* __restrict__ q, const E* __restrict__ rows, int bs,
+                                                  const int32_t* __restrict__ block_tables, int bt_width,
+                                                  const int32_t* __restrict__ seq_of, const int64_t* __restrict__ pos,
+                                                  float scale, const float* __restrict__ talk, const E* __restrict__ gate,
+                                                  int64_t g_st, E* __restrict__ out, float* __restrict__ part, int nsplit,
+                                                  int H, int G, int d, int KT) {
+  extern __shared__ float lds[];
+  const int t = blockIdx.x, sp = blockIdx.y, tid = threadIdx.x;
+  const int wv = tid >> 6, lane = tid & 63;
+  const int Hd = H * d, Gd = G * d, KP = KT + 1;
+  const int JS = Gd >= 256 ? 1 : 256 / Gd;
+  constexpr int per = Words<E>::per;
+  const int row_w = 2 * Gd / per;                   // words per cache row
+  const int pitch = row_w | 1;                      // odd word pitch: conflict-free column walks
+  float* qs = lds;
+  float* tk = qs + Hd;
+  float* S = tk + H * H;
+  float* S2 = S + H * KP;
+  float* mrun = S2 + H * KP;
+  float* lrun = mrun + H;
+  float* corr = lrun + H;
+  float* red = corr + H;
+  uint32_t* tile = (uint32_t*)(red + JS * Hd);
+
+  const int64_t L = pos[t] + 1;                     // keys this token sees
+  const int b = seq_of[t];
+  const int32_t* bt = block_tables + (int64_t)b * bt_width;
+  const int64_t tiles_total = (L + KT - 1) / KT;
+  const int64_t tiles_per = (tiles_total + nsplit - 1) / nsplit;
+  const int64_t k_lo = (int64_t)sp * tiles_per * KT;
+  const int64_t k_hi = L < k_lo + tiles_per * KT ? L : k_lo + tiles_per * KT;
+
+  for (int i = tid; i < Hd; i += 256) qs[i] = q[(int64_t)t * Hd + i];
+  for (int i = tid; i < H * H; i += 256) tk[i] = talk ? talk[i] : ((i / H) == (i % H) ? 1.f : 0.f);
+  if (tid < H) {
+    mrun[tid] = -INFINITY;
+    lrun[tid] = 0.f;
+    corr[tid] = 0.f;
+  }
+  float acc[kMaxItems][REP];
+#pragma unroll
+  for (int a = 0; a < kMaxItems; a++)
+#pragma unroll
+    for (int r = 0; r < REP; r++) acc[a][r] = 0.f;
+  const int js = JS > 1 ? tid / Gd : 0;
+  const bool pv_on = JS > 1 ? tid < JS * Gd : true;
+  __syncthreads();
+
+  for (int64_t j0 = k_lo; j0 < k_hi; j0 += KT) {
+    const int nv = (int)(k_hi - j0 < KT ? k_hi - j0 : KT);
+    // ---- tile load: 16-byte pieces of the nv rows
+    {
+      const int pieces = row_w / 4;                 // row_w is a multiple of 4 words (d % 8 == 0)
+      for (int i = tid; i < nv * pieces; i += 256) {
+        const int j = i / pieces, c = i - j * pieces;
+        const int64_t kp = j0 + j;
+        const int64_t row = (int64_t)bt[kp / bs] * bs + kp % bs;
+        const uint4 v = *(const uint4*)((const uint32_t*)rows + row * row_w + c * 4);
+        uint32_t* dst = tile + j * pitch + c * 4;
+        dst[0] = v.x;
+        dst[1] = v.y;
+        dst[2] = v.z;
+        dst[3] = v.w;
+      }
+    }
+    __syncthreads();
+    // ---- scores: item (key j, kv head g) -> REP heads
+    for (int it = tid; it < KT * G; it += 256) {
+      const int j = it % KT, g = it / KT;
+      if (j < nv) {
+        float a[REP];
+#pragma unroll
+        for (int r = 0; r < REP; r++) a[r] = 0.f;
+        const uint32_t* kr = tile + j * pitch + g * d / per;
+        const float* qg = qs + g * REP * d;
+        for (int i = 0; i < d / per; i++) {
+          float kv[2];
+          Words<E>::get(kr[i], kv);
+#pragma unroll
+          for (int r = 0; r < REP; r++) {
+#pragma unroll
+            for (int e = 0; e < per; e++) a[r] += qg[r * d + i * per + e] * kv[e];
+          }
+        }
+#pragma unroll
+        for (int r = 0; r < REP; r++) S[(g * REP + r) * KP + j] = a[r] * scale;
+      }
+    }
+    __syncthreads();
+    // ---- mixing over the heads + mask
+    for (int it = tid; it < KT * H; it += 256) {
+      const int j = it % KT, h = it / KT;
+      float v = -INFINITY;
+      if (j < nv) {
+        v = 0.f;
+        for (int g = 0; g < H; g++) v += tk[h * H + g] * S[g * KP + j];
+      }
+      S2[h * KP + j] = v;
+    }
+    __syncthreads();
+    // ---- online softmax: a wave per head in turn; weights go to S
+    for (int h = wv; h < H; h += 4) {
+      float mt = -INFINITY;
+      for (int j = lane; j < KT; j += 64) mt = fmaxf(mt, S2[h * KP + j]);
+      mt = wave_max(mt);
+      const float mo = mrun[h], mn = fmaxf(mo, mt);
+      float ls = 0.f;
+      for (int j = lane; j < KT; j += 64) {
+        const float pj = j < nv ? expf(S2[h * KP + j] - mn) : 0.f;
+        S[h * KP + j] = pj;
+        ls += pj;
+      }
+      ls = wave_sum(ls);
+      if (lane == 0) {
+        const float c = expf(mo - mn);              // mo = -inf at the first tile: 0
+        corr[h] = c;
+        lrun[h] = lrun[h] * c + ls;
+        mrun[h] = mn;
+      }
+    }
+    __syncthreads();
+    // ---- weighted sum of the values
+    if (pv_on) {
+#pragma unroll
+      for (int a = 0; a < kMaxItems; a++) {
+        const int item = JS > 1 ? tid - js * Gd : tid + a * 256;
+        if ((JS > 1 && a > 0) || item >= Gd) break;
+        const int g = item / d;
+#pragma unroll
+        for (int r = 0; r < REP; r++) acc[a][r] *= corr[g * REP + r];
+        const E* vcol = (const E*)tile + Gd + item;
+        for (int j = js; j < nv; j += JS) {
+          const float v = ldf(vcol + (int64_t)j * pitch * per);
+#pragma unroll
+          for (int r = 0; r < REP; r++) acc[a][r] += S[(g * REP + r) * KP + j] * v;
+        }
+      }
+    }
+    __syncthreads();
+  }
+  // ---- partial sums of the key-interleaved thread groups -> red [JS][H d]
+  if (pv_on) {
+#pragma unroll
+    for (int a = 0; a < kMaxItems; a++) {
+      const int item = JS > 1 ? tid - js * Gd : tid + a * 256;
+      if ((JS > 1 && a > 0) || item >= Gd) break;
+      const int g = item / d, c = item - g * d;
+#pragma unroll
+      for (int r = 0; r < REP; r++) red[js * Hd + (g * REP + r) * d + c] = acc[a][r];
+    }
+  }
+  __syncthreads();
+  for (int o = tid; o < Hd; o += 256) {
+    const int h = o / d, c = o - h * d;
+    float v = 0.f;
+    for (int s = 0; s < JS; s++) v += red[s * Hd + o];
+    if (nsplit == 1) {
+      v /= lrun[h];
+      if (gate) v *= 1.0f / (1.0f + expf(-ldf(gate + (int64_t)t * g_st + o)));
+      stf(out + (int64_t)t * Hd + o, v);
+    } else {
+      float* pr = part + (((int64_t)t * nsplit + sp) * H + h) * (d + 2);
+      pr[c] = v;
+      if (c == 0) {
+        pr[d] = mrun[h];
+        pr[d + 1] = lrun[h];
+      }
+    }
+  }
+}
+
+template <typename E>
+__global__ void __launch_bounds__(256) talk_attn_combine_k(const float* __restrict__ part, const E* __restrict__ gate,
+                                                          int64_t g_st, E* __restrict__ out, int nsplit, int H, int d) {
+  const int64_t t = blockIdx.x;
+  const int Hd = H * d;
+  for (int o = threadIdx.x; o < Hd; o += blockDim.x) {
+    const int h = o / d, c = o - h * d;
+    const float* pr = part + ((int64_t)t * nsplit * H + h) * (d + 2);
+    const int64_t st = (int64_t)H * (d + 2);
+    float M = -INFINITY;
+    for (int s = 0; s < nsplit; s++) M = fmaxf(M, pr[s * st + d]);
+    float l = 0.f, v = 0.f;
+    for (int s = 0; s < nsplit; s++) {
+      const float m = pr[s * st + d];
+      if (m == -INFINITY) continue;               // an empty split
+      const float e = expf(m - M);
+      l += pr[s * st + d + 1] * e;
+      v += pr[s * st + c] * e;
+    }
+    v /= l;
+    if (gate) v *= 1.0f / (1.0f + expf(-ldf(gate + t * g_st + o)));
+    stf(out + t * Hd + o, v);
+  }
+}
+
+// ------------------------------------------------------------------ softmax step of the library-product path
+// one block per token: rows t H .. t H + H - 1 of sc [nt H, L].  Pass A mixes the H raw scores of every key
+// column (scaled) in place; pass B is the masked softmax of every row, a wave per row in turn.
+template <typename E, int HM>
+__global__ void __launch_bounds__(256) talk_softmax_k(float* __restrict__ sc, const int64_t* __restrict__ pos, int H,
+                                                     float scale, const float* __restrict__ talk, int L,
+                                                     E* __restrict__ hi, E* __restrict__ lo) {
+  __shared__ float tk[HM * HM];
+  const int64_t t = blockIdx.x;
+  const int tid = threadIdx.x, wv = tid >> 6, lane = tid & 63;
+  float* base = sc + t * H * (int64_t)L;
+  int64_t nk = pos[t] + 1;
+  if (nk > L) nk = L;
+  if (nk < 0) nk = 0;
+  if (talk) {
+    for (int i = tid; i < H * H; i += 256) tk[i] = talk[i] * scale;
+    __syncthreads();
+    for (int j = tid; j < nk; j += 256) {
+      float s[HM];
+#pragma unroll
+      for (int g = 0; g < HM; g++) s[g] = g < H ? base[(int64_t)g * L + j] : 0.f;
+#pragma unroll
+      for (int h = 0; h < HM; h++) {
+        if (h < H) {
+          float v = 0.f;
+#pragma unroll
+          for (int g = 0; g < HM; g++)
+            if (g < H) v += tk[h * H + g] * s[g];
+          base[(int64_t)h * L + j] = v;
+        }
+      }
+    }
+    __syncthreads();
+  }
+  const float post = talk ? 1.0f : scale;
+  for (int h = wv; h < H; h += 4) {
+    float* r = base + (int64_t)h * L;
+    float m = -INFINITY;
+    for (int j = lane; j < nk; j += 64) m = fmaxf(m, r[j] * post);
+    m = wave_max(m);
+    float l = 0.f;
+    for (int j = lane; j < nk; j += 64) l += expf(r[j] * post - m);
+    l = wave_sum(l);
+    const float inv = 1.0f / l;
+    for (int j = lane; j < L; j += 64) {
+      const float p = j < nk ? expf(r[j] * post - m) * inv : 0.f;
+      if (hi) {
+        const __bf16 ph = (__bf16)p;
+        const int64_t o = (t * H + h) * (int64_t)L + j;
+        ((__bf16*)hi)[o] = ph;
+        ((__bf16*)lo)[o] = (__bf16)(p - (float)ph);
+      } else {
+        r[j] = p;
+      }
+    }
+  }
+}
+
+int lds_floats(int H, int G, int d, int KT) {
+  const int Gd = G * d, JS = Gd >= 256 ? 1 : 256 / Gd;
+  return H * d + H * H + 2 * H * (KT + 1) + 3 * H + JS * H * d;
+}
+
+}  // namespace
+
+void qk_norm_rope_store(bool bf16, const void* q, int64_t q_ld, const void* k, int64_t k_ld, const void* qn,
+                        const void* kn, float eps, const float* table, int max_pos, int dims, const int64_t* pos,
+                        const int64_t* slots, void* rows, int64_t num_rows, float* qo, int T, int H, int G, int d,
+                        hipStream_t st) {
+  if (T <= 0) return;
+  const size_t lds = (size_t)4 * d * sizeof(float);
+  if (bf16)
+    qk_norm_rope_store_k<__bf16><<<T, 256, lds, st>>>((const __bf16*)q, q_ld, (const __bf16*)k, k_ld, (const __bf16*)qn,
+                                                      (const __bf16*)kn, eps, table, max_pos, dims, pos, slots,
+                                                      (__bf16*)rows, num_rows, qo, H, G, d);
+  else
+    qk_norm_rope_store_k<float><<<T, 256, lds, st>>>((const float*)q, q_ld, (const float*)k, k_ld, (const float*)qn,
+                                                     (const float*)kn, eps, table, max_pos, dims, pos, slots,
+                                                     (float*)rows, num_rows, qo, H, G, d);
+}
+
+int talk_attention_plan(bool bf16, int H, int G, int d, int* kt) {
+  if (H < 1 || G < 1 || H % G || d < 8 || d % 8 || G * d > 256 * kMaxItems) return -1;
+  const int rep = H / G;
+  if (rep > 8) return -1;
+  const int per = bf16 ? 2 : 1;
+  const int pitch = (2 * G * d / per) | 1;
+  for (int KT = 64; KT >= 8; KT >>= 1) {
+    const int64_t bytes = (int64_t)lds_floats(H, G, d, KT) * 4 + (int64_t)KT * pitch * 4;
+    if (bytes <= 64 * 1024) {
+      *kt = KT;
+      return (int)bytes;
+    }
+  }
+  return -1;
+}
+
+int talk_attention_splits(bool bf16, int T, int H, int G, int d, int max_ctx) {
+  int kt = 0;
+  if (talk_attention_plan(bf16, H, G, d, &kt) < 0) return 1;
+  const int tiles = (max_ctx + kt - 1) / kt;
+  int ns = 1;
+  // fill the chip (256 CUs, a few workgroups each), at least 4 tiles per split
+  while (ns < 64 && (int64_t)T * ns < 1024 && tiles / (ns * 2) >= 4) ns *= 2;
+  return ns;
+}
+
+template <typename E, int REP>
+static void launch_talk(const float* q, const void* rows, int bs, const int32_t* bt, int btw, const int32_t* seq_of,
+                        const int64_t* pos, float scale, const float* talk, const void* gate, int64_t g_st, void* out,
+                        float* part, int nsplit, int T, int H, int G, int d, int KT, int lds, hipStream_t st) {
+  talk_attn_k<E, REP><<<dim3(T, nsplit), 256, lds, st>>>(q, (const E*)rows, bs, bt, btw, seq_of, pos, scale, talk,
+                                                          (const E*)gate, g_st, (E*)out, part, nsplit, H, G, d, KT);
+}
+
+void talk_attention(bool bf16, const float* q, const void* rows, int bs, const int32_t* block_tables, int bt_width,
+                    const int32_t* seq_of, const int64_t* pos, float scale, const float* talk, const void* gate,
+                    int64_t g_st, void* out, float* part, int nsplit, int T, int H, int G, int d, hipStream_t st) {
+  if (T <= 0) return;
+  int KT = 0;
+  const int lds = talk_attention_plan(bf16, H, G, d, &KT);
+  if (lds < 0) return;                              // callers check the plan first
+#define BM_REP(R)                                                                                                     \
+  case R:                                                                                                             \
+    if (bf16) launch_talk<__bf16, R>(q, rows, bs, block_tables, bt_width, seq_of, pos, scale, talk, gate, g_st, out,  \
+                                     part, nsplit, T, H, G, d, KT, lds, st);                                          \
+    else launch_talk<float, R>(q, rows, bs, block_tables, bt_width, seq_of, pos, scale, talk, gate, g_st, out, part,  \
+                               nsplit, T, H, G, d, KT, lds, st);                                                      \
+    break;
+  switch (H / G) {
+    BM_REP(1) BM_REP(2) BM_REP(3) BM_REP(4) BM_REP(5) BM_REP(6) BM_REP(7) BM_REP(8)
+    default: return;
+  }
+#undef BM_REP
+  if (nsplit > 1) {
+    if (bf16) talk_attn_combine_k<__bf16><<<T, 256, 0, st>>>(part, (const __bf16*)gate, g_st, (__bf16*)out, nsplit, H, d);
+    else talk_attn_combine_k<float><<<T, 256, 0, st>>>(part, (const float*)gate, g_st, (float*)out, nsplit, H, d);
+  }
+}
+
+void talk_softmax(bool bf16, float* sc, const int64_t* pos, int H, float scale, const float* talk, int64_t nt, int L,
+                  void* hi, void* lo, hipStream_t st) {
+  if (nt <= 0) return;
+#define BM_HM(HM)                                                                                                  \
+  if (bf16) talk_softmax_k<__bf16, HM><<<nt, 256, 0, st>>>(sc, pos, H, scale, talk, L, (__bf16*)hi, (__bf16*)lo);   \
+  else talk_softmax_k<float, HM><<<nt, 256, 0, st>>>(sc, pos, H, scale, talk, L, (float*)nullptr, (float*)nullptr);
+  if (H <= 8) { BM_HM(8) }
+  else if (H <= 16) { BM_HM(16) }
+  else if (H <= 32) { BM_HM(32) }
+  else { BM_HM(64) }
+#undef BM_HM
+}
+
+}  // namespace bm
+}  // namespace illm

@@ -55,9 +55,11 @@ class HybridCache:
 
     ``layer_specs[i]`` is ``("rows", width)`` for a layer that appends one
     ``width``-wide row per token to a paged pool (a latent-attention layer
-    keeps ``[latent | rotated key]``), ``("state", {name: shape})`` for a layer
-    with per-sequence f32 state tensors (``shape`` without the slot axis), or
-    ``None``.  Row pools are ``[num_blocks + 1, block_size, width]`` and state
+    keeps ``[latent | rotated key]``, a grouped-attention layer ``[keys |
+    values]``), ``("state", {name: shape})`` for a layer with per-sequence f32
+    state tensors (``shape`` without the slot axis), ``None``, or a list of
+    such entries for a layer that has both (paged rows and, say, the last
+    inputs of a short convolution).  Row pools are ``[num_blocks + 1, block_size, width]`` and state
     pools ``[num_slots + 1, *shape]``: the last block / slot is a scratch
     target for padded batch rows.  ``k`` / ``v`` alias the row pools so the
     engines' device probes (``cache.k[0]``) keep working."""
@@ -72,13 +74,17 @@ class HybridCache:
         self.device = torch.device(device)
         self.rows: List[Optional[torch.Tensor]] = []
         self.state: List[Optional[dict]] = []
-        for spec in layer_specs:
+        for entry in layer_specs:
             rows, st = None, None
-            if spec is not None and spec[0] == "rows":
-                rows = torch.zeros(num_blocks + 1, block_size, int(spec[1]), dtype=dtype, device=device)
-            elif spec is not None and spec[0] == "state":
-                st = {n: torch.zeros(num_slots + 1, *shape, dtype=torch.float32, device=device)
-                      for n, shape in spec[1].items()}
+            for spec in (entry if isinstance(entry, list) else [entry]):
+                if spec is not None and spec[0] == "rows":
+                    if rows is not None:
+                        raise ValueError("one paged row pool per layer")
+                    rows = torch.zeros(num_blocks + 1, block_size, int(spec[1]), dtype=dtype, device=device)
+                elif spec is not None and spec[0] == "state":
+                    st = dict(st or {})
+                    st.update({n: torch.zeros(num_slots + 1, *shape, dtype=torch.float32, device=device)
+                               for n, shape in spec[1].items()})
             self.rows.append(rows)
             self.state.append(st)
         probe = next((r for r in self.rows if r is not None), None)

@@ -17,6 +17,7 @@ import torch
 
 NATIVE_ARCHITECTURES = {
     "Zamelix": "ipex_llm_amd.models.zamelix",
+    "Masezen": "ipex_llm_amd.models.masezen",
 }
 
 
