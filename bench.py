@@ -164,7 +164,18 @@ def main():
     ap.add_argument("--hybrid-sizes", default="small,base")
     ap.add_argument("--hybrid-prompts", default="1024,4096")
     ap.add_argument("--no-hybrid-ref", action="store_true", help="--hybrid: skip the MLA comparison model")
+    ap.add_argument("--blockmix", action="store_true",
+                    help="side benchmark (not the headline metric): prefill / decode throughput of the parallel-residual "
+                         "decoder (grouped attention with mixed head scores; dense and expert feed-forward) beside the "
+                         "Qwen3-style grouped-query decoder at equal sizes, one GPU")
+    ap.add_argument("--blockmix-sizes", default="small,base")
+    ap.add_argument("--blockmix-prompts", default="1024,4096")
+    ap.add_argument("--no-blockmix-ref", action="store_true", help="--blockmix: skip the comparison model")
     args = ap.parse_args()
+    if args.blockmix:
+        from ipex_llm_amd.utils.bench_blockmix import main as blockmix_main
+        blockmix_main(args)
+        return
     if args.hybrid:
         from ipex_llm_amd.utils.bench_hybrid import main as hybrid_main
         hybrid_main(args)

@@ -112,9 +112,17 @@ template <> struct Words<__bf16> {
   }
 };
 
-// LDS layout (floats unless noted): qs [H d] | tk [H H] | S [H (KT + 1)] | S2 [H (KT + 1)] | mrun lrun corr [3 H] |
-// red [JS H d] | tile (uint32 words) [KT pitch_w]
-template <typename E, int REP>
+typedef __bf16 bm_bf16x8 __attribute__((ext_vector_type(8)));
+typedef float bm_f32x4 __attribute__((ext_vector_type(4)));
+
+__host__ __device__ __forceinline__ int round4(int n) { return (n + 3) & ~3; }
+
+// LDS layout (floats unless noted, every region a multiple of 16 bytes): qs [H (d + 8)] | tk [H H] | S [H (KT + 1)] |
+// S2 [H (KT + 1)] | mrun lrun corr [3 H] | red [JS H d] | tile (uint32 words) [KT pitch_w].
+// MF (bf16 rows, d a multiple of 32): the scores run on the matrix cores -- 16 keys x 16 (padded) heads of one
+// key / value head per 16x16x32 MFMA, the f32 queries split into bf16 hi + lo halves (qs then holds those, rows of
+// d + 8) -- and the tile rows are 16-byte aligned; otherwise vector FMAs over rows of an odd word pitch.
+template <typename E, int REP, bool MF>
 __global__ void __launch_bounds__(256) talk_attn_k(const float* __restrict__ q, const E* __restrict__ rows, int bs,
                                                   const int32_t* __restrict__ block_tables, int bt_width,
                                                   const int32_t* __restrict__ seq_of, const int64_t* __restrict__ pos,
@@ -128,16 +136,17 @@ __global__ void __launch_bounds__(256) talk_attn_k(const float* __restrict__ q, 
   const int JS = Gd >= 256 ? 1 : 256 / Gd;
   constexpr int per = Words<E>::per;
   const int row_w = 2 * Gd / per;                   // words per cache row
-  const int pitch = row_w | 1;                      // odd word pitch: conflict-free column walks
+  const int pitch = MF ? row_w + 4 : (row_w | 1);   // aligned rows for MFMA operands, else an odd word pitch
+  const int DP = d + 8;
   float* qs = lds;
-  float* tk = qs + Hd;
-  float* S = tk + H * H;
-  float* S2 = S + H * KP;
-  float* mrun = S2 + H * KP;
+  float* tk = qs + round4(H * DP);
+  float* S = tk + round4(H * H);
+  float* S2 = S + round4(H * KP);
+  float* mrun = S2 + round4(H * KP);
   float* lrun = mrun + H;
   float* corr = lrun + H;
-  float* red = corr + H;
-  uint32_t* tile = (uint32_t*)(red + JS * Hd);
+  float* red = mrun + round4(3 * H);
+  uint32_t* tile = (uint32_t*)(red + round4(JS * Hd));
 
   const int64_t L = pos[t] + 1;                     // keys this token sees
   const int b = seq_of[t];
@@ -147,7 +156,19 @@ __global__ void __launch_bounds__(256) talk_attn_k(const float* __restrict__ q, 
   const int64_t k_lo = (int64_t)sp * tiles_per * KT;
   const int64_t k_hi = L < k_lo + tiles_per * KT ? L : k_lo + tiles_per * KT;
 
-  for (int i = tid; i < Hd; i += 256) qs[i] = q[(int64_t)t * Hd + i];
+  if (MF) {
+    __bf16* qh = (__bf16*)qs;
+    __bf16* ql = qh + H * DP;
+    for (int i = tid; i < Hd; i += 256) {
+      const int h = i / d, c = i - h * d;
+      const float v = q[(int64_t)t * Hd + i];
+      const __bf16 hi = (__bf16)v;
+      qh[h * DP + c] = hi;
+      ql[h * DP + c] = (__bf16)(v - (float)hi);
+    }
+  } else {
+    for (int i = tid; i < Hd; i += 256) qs[i] = q[(int64_t)t * Hd + i];
+  }
   for (int i = tid; i < H * H; i += 256) tk[i] = talk ? talk[i] : ((i / H) == (i % H) ? 1.f : 0.f);
   if (tid < H) {
     mrun[tid] = -INFINITY;
@@ -174,14 +195,48 @@ __global__ void __launch_bounds__(256) talk_attn_k(const float* __restrict__ q, 
         const int64_t row = (int64_t)bt[kp / bs] * bs + kp % bs;
         const uint4 v = *(const uint4*)((const uint32_t*)rows + row * row_w + c * 4);
         uint32_t* dst = tile + j * pitch + c * 4;
-        dst[0] = v.x;
-        dst[1] = v.y;
-        dst[2] = v.z;
-        dst[3] = v.w;
+        if (MF) {
+          *(uint4*)dst = v;
+        } else {
+          dst[0] = v.x;
+          dst[1] = v.y;
+          dst[2] = v.z;
+          dst[3] = v.w;
+        }
       }
     }
     __syncthreads();
-    // ---- scores: item (key j, kv head g) -> REP heads
+    // ---- scores
+    if (MF) {
+      const int r16 = lane & 15, gq = lane >> 4;
+      const __bf16* qh = (const __bf16*)qs;
+      const __bf16* ql = qh + H * DP;
+      const int nchunk = (nv + 15) >> 4;
+      const bool hv = r16 < REP;
+      const bm_bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+      for (int u = wv; u < G * nchunk; u += 4) {
+        const int g = u / nchunk, kc = u - g * nchunk;
+        const int h = g * REP + (hv ? r16 : 0);
+        const __bf16* ka = (const __bf16*)tile + (int64_t)(kc * 16 + r16) * pitch * 2 + g * d + 8 * gq;
+        const __bf16* qa = qh + h * DP + 8 * gq;
+        const __bf16* qb = ql + h * DP + 8 * gq;
+        bm_f32x4 a4 = {0.f, 0.f, 0.f, 0.f};
+        for (int ks = 0; ks < d / 32; ks++) {
+          const bm_bf16x8 a = *(const bm_bf16x8*)(ka + 32 * ks);
+          const bm_bf16x8 bh = hv ? *(const bm_bf16x8*)(qa + 32 * ks) : zero8;
+          const bm_bf16x8 bl = hv ? *(const bm_bf16x8*)(qb + 32 * ks) : zero8;
+          a4 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, bh, a4, 0, 0, 0);
+          a4 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, bl, a4, 0, 0, 0);
+        }
+        if (hv) {
+#pragma unroll
+          for (int i = 0; i < 4; i++) {
+            const int key = kc * 16 + 4 * gq + i;     // lane: keys 4 gq + i of head r16
+            if (key < KT) S[h * KP + key] = a4[i] * scale;
+          }
+        }
+      }
+    } else
     for (int it = tid; it < KT * G; it += 256) {
       const int j = it % KT, g = it / KT;
       if (j < nv) {
@@ -286,28 +341,32 @@ __global__ void __launch_bounds__(256) talk_attn_k(const float* __restrict__ q, 
   }
 }
 
+// one block per (token, head): the splits' maxima and sums by the first wave, then a thread per value column
 template <typename E>
-__global__ void __launch_bounds__(256) talk_attn_combine_k(const float* __restrict__ part, const E* __restrict__ gate,
+__global__ void __launch_bounds__(128) talk_attn_combine_k(const float* __restrict__ part, const E* __restrict__ gate,
                                                           int64_t g_st, E* __restrict__ out, int nsplit, int H, int d) {
+  __shared__ float wgt[64];
+  __shared__ float linv;
   const int64_t t = blockIdx.x;
-  const int Hd = H * d;
-  for (int o = threadIdx.x; o < Hd; o += blockDim.x) {
-    const int h = o / d, c = o - h * d;
-    const float* pr = part + ((int64_t)t * nsplit * H + h) * (d + 2);
-    const int64_t st = (int64_t)H * (d + 2);
-    float M = -INFINITY;
-    for (int s = 0; s < nsplit; s++) M = fmaxf(M, pr[s * st + d]);
-    float l = 0.f, v = 0.f;
-    for (int s = 0; s < nsplit; s++) {
-      const float m = pr[s * st + d];
-      if (m == -INFINITY) continue;               // an empty split
-      const float e = expf(m - M);
-      l += pr[s * st + d + 1] * e;
-      v += pr[s * st + c] * e;
-    }
-    v /= l;
+  const int h = blockIdx.y, tid = threadIdx.x;
+  const float* pr = part + ((int64_t)t * nsplit * H + h) * (d + 2);
+  const int64_t st = (int64_t)H * (d + 2);
+  if (tid < 64) {
+    const float m = tid < nsplit ? pr[tid * st + d] : -INFINITY;
+    const float M = wave_max(m);
+    const float e = m == -INFINITY ? 0.f : expf(m - M);       // an empty split weighs nothing
+    const float l = wave_sum(tid < nsplit ? pr[tid * st + d + 1] * e : 0.f);
+    wgt[tid] = e;
+    if (tid == 0) linv = 1.0f / l;
+  }
+  __syncthreads();
+  for (int c = tid; c < d; c += 128) {
+    float v = 0.f;
+    for (int s = 0; s < nsplit; s++) v += pr[s * st + c] * wgt[s];
+    v *= linv;
+    const int o = h * d + c;
     if (gate) v *= 1.0f / (1.0f + expf(-ldf(gate + t * g_st + o)));
-    stf(out + t * Hd + o, v);
+    stf(out + t * (int64_t)H * d + o, v);
   }
 }
 
@@ -371,8 +430,10 @@ __global__ void __launch_bounds__(256) talk_softmax_k(float* __restrict__ sc, co
 
 int lds_floats(int H, int G, int d, int KT) {
   const int Gd = G * d, JS = Gd >= 256 ? 1 : 256 / Gd;
-  return H * d + H * H + 2 * H * (KT + 1) + 3 * H + JS * H * d;
+  return round4(H * (d + 8)) + round4(H * H) + 2 * round4(H * (KT + 1)) + round4(3 * H) + round4(JS * H * d);
 }
+
+bool use_mfma(bool bf16, int d) { return bf16 && d % 32 == 0; }
 
 }  // namespace
 
@@ -397,8 +458,9 @@ int talk_attention_plan(bool bf16, int H, int G, int d, int* kt) {
   const int rep = H / G;
   if (rep > 8) return -1;
   const int per = bf16 ? 2 : 1;
-  const int pitch = (2 * G * d / per) | 1;
-  for (int KT = 64; KT >= 8; KT >>= 1) {
+  const bool mf = use_mfma(bf16, d);
+  const int pitch = mf ? 2 * G * d / per + 4 : ((2 * G * d / per) | 1);
+  for (int KT = 64; KT >= (mf ? 16 : 8); KT >>= 1) {
     const int64_t bytes = (int64_t)lds_floats(H, G, d, KT) * 4 + (int64_t)KT * pitch * 4;
     if (bytes <= 64 * 1024) {
       *kt = KT;
@@ -414,15 +476,15 @@ int talk_attention_splits(bool bf16, int T, int H, int G, int d, int max_ctx) {
   const int tiles = (max_ctx + kt - 1) / kt;
   int ns = 1;
   // fill the chip (256 CUs, a few workgroups each), at least 4 tiles per split
-  while (ns < 64 && (int64_t)T * ns < 1024 && tiles / (ns * 2) >= 4) ns *= 2;
+  while (ns < 64 && (int64_t)T * ns < 512 && tiles / (ns * 2) >= 4) ns *= 2;
   return ns;
 }
 
-template <typename E, int REP>
+template <typename E, int REP, bool MF>
 static void launch_talk(const float* q, const void* rows, int bs, const int32_t* bt, int btw, const int32_t* seq_of,
                         const int64_t* pos, float scale, const float* talk, const void* gate, int64_t g_st, void* out,
                         float* part, int nsplit, int T, int H, int G, int d, int KT, int lds, hipStream_t st) {
-  talk_attn_k<E, REP><<<dim3(T, nsplit), 256, lds, st>>>(q, (const E*)rows, bs, bt, btw, seq_of, pos, scale, talk,
+  talk_attn_k<E, REP, MF><<<dim3(T, nsplit), 256, lds, st>>>(q, (const E*)rows, bs, bt, btw, seq_of, pos, scale, talk,
                                                           (const E*)gate, g_st, (E*)out, part, nsplit, H, G, d, KT);
 }
 
@@ -435,9 +497,13 @@ void talk_attention(bool bf16, const float* q, const void* rows, int bs, const i
   if (lds < 0) return;                              // callers check the plan first
 #define BM_REP(R)                                                                                                     \
   case R:                                                                                                             \
-    if (bf16) launch_talk<__bf16, R>(q, rows, bs, block_tables, bt_width, seq_of, pos, scale, talk, gate, g_st, out,  \
-                                     part, nsplit, T, H, G, d, KT, lds, st);                                          \
-    else launch_talk<float, R>(q, rows, bs, block_tables, bt_width, seq_of, pos, scale, talk, gate, g_st, out, part,  \
+    if (bf16 && use_mfma(true, d))                                                                                    \
+      launch_talk<__bf16, R, true>(q, rows, bs, block_tables, bt_width, seq_of, pos, scale, talk, gate, g_st, out,    \
+                                   part, nsplit, T, H, G, d, KT, lds, st);                                            \
+    else if (bf16)                                                                                                    \
+      launch_talk<__bf16, R, false>(q, rows, bs, block_tables, bt_width, seq_of, pos, scale, talk, gate, g_st, out,   \
+                                    part, nsplit, T, H, G, d, KT, lds, st);                                           \
+    else launch_talk<float, R, false>(q, rows, bs, block_tables, bt_width, seq_of, pos, scale, talk, gate, g_st, out, part,  \
                                nsplit, T, H, G, d, KT, lds, st);                                                      \
     break;
   switch (H / G) {
@@ -446,8 +512,10 @@ void talk_attention(bool bf16, const float* q, const void* rows, int bs, const i
   }
 #undef BM_REP
   if (nsplit > 1) {
-    if (bf16) talk_attn_combine_k<__bf16><<<T, 256, 0, st>>>(part, (const __bf16*)gate, g_st, (__bf16*)out, nsplit, H, d);
-    else talk_attn_combine_k<float><<<T, 256, 0, st>>>(part, (const float*)gate, g_st, (float*)out, nsplit, H, d);
+    if (bf16)
+      talk_attn_combine_k<__bf16><<<dim3(T, H), 128, 0, st>>>(part, (const __bf16*)gate, g_st, (__bf16*)out, nsplit, H, d);
+    else
+      talk_attn_combine_k<float><<<dim3(T, H), 128, 0, st>>>(part, (const float*)gate, g_st, (float*)out, nsplit, H, d);
   }
 }
 

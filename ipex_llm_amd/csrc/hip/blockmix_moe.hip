@@ -10,8 +10,9 @@
 //                  GLU form: x = w_pair * h[token] (rounded to the activation
 //                  type), y = g sigmoid(alpha g) (u + 1) with the clamps;
 //                  DOWN form: f32 rows scattered back by pair id.
-//                  bf16: 16x16x16 MFMA tiles with f32 accumulation; f32:
-//                  vector FMAs.  A row's sum runs over k in one fixed order,
+//                  bf16: 16x16x32 MFMA tiles with f32 accumulation
+//                  (moe_gemm_mfma_k); f32, and sizes that are no multiple of
+//                  8: vector FMAs.  A row's sum runs over k in one fixed order,
 //                  so a token's result does not depend on its batch.
 #include "blockmix.h"
 
@@ -104,16 +105,17 @@ __global__ void __launch_bounds__(1024) moe_align_k(const int32_t* __restrict__ 
 
 constexpr int TM = 32, TN = 64, TK = 32;
 
-// which (expert, row block) this workgroup serves; false: past the last one
-__device__ __forceinline__ bool find_block(const int32_t* __restrict__ off, int E, int bx, int* e_out, int* r0, int* r1) {
+// which (expert, block of tm rows) this workgroup serves; false: past the last one
+__device__ __forceinline__ bool find_block(const int32_t* __restrict__ off, int E, int bx, int tm, int* e_out, int* r0,
+                                           int* r1) {
   int acc = 0;
   for (int e = 0; e < E; e++) {
     const int lo = off[e], hi = off[e + 1];
-    const int nb = (hi - lo + TM - 1) / TM;
+    const int nb = (hi - lo + tm - 1) / tm;
     if (bx < acc + nb) {
       *e_out = e;
-      *r0 = lo + (bx - acc) * TM;
-      *r1 = hi < *r0 + TM ? hi : *r0 + TM;
+      *r0 = lo + (bx - acc) * tm;
+      *r1 = hi < *r0 + tm ? hi : *r0 + tm;
       return true;
     }
     acc += nb;
@@ -135,7 +137,7 @@ __global__ void __launch_bounds__(256) moe_gemm_k(const E* __restrict__ x, const
   __shared__ float src_scale[TM];
   __shared__ int dst_row[TM];
   int e, r0, r1;
-  if (!find_block(off, nexp, blockIdx.x, &e, &r0, &r1)) return;
+  if (!find_block(off, nexp, blockIdx.x, TM, &e, &r0, &r1)) return;
   const int tid = threadIdx.x;
   const int n0 = blockIdx.y * TN;
   if (tid < TM) {
@@ -217,6 +219,103 @@ __global__ void __launch_bounds__(256) moe_gemm_k(const E* __restrict__ x, const
   }
 }
 
+
+// ---- bf16 on the matrix cores: 16x16x32 MFMA tiles, f32 accumulation.  A workgroup serves TMM gathered rows x 64
+// columns; wave w owns columns 16 w .. 16 w + 15 and reads its weight fragments straight from memory (every weight
+// element is used by exactly one wave of the workgroup, for all its row tiles); the gathered, scaled rows go through LDS.
+typedef __bf16 bm_bf16x8 __attribute__((ext_vector_type(8)));
+typedef float bm_f32x4 __attribute__((ext_vector_type(4)));
+
+template <int TMM, bool GLU>
+__global__ void __launch_bounds__(256) moe_gemm_mfma_k(const __bf16* __restrict__ x, const int32_t* __restrict__ off,
+                                                      const int32_t* __restrict__ sorted, const float* __restrict__ wts,
+                                                      int top, const __bf16* __restrict__ w, __bf16* __restrict__ y,
+                                                      float* __restrict__ outp, int nexp, int N, int K, float limit,
+                                                      float alpha) {
+  constexpr int TKK = 64, AP = TKK + 8, MS = TMM / 16;
+  __shared__ __attribute__((aligned(16))) __bf16 as[TMM * AP];
+  __shared__ int src_row[TMM];
+  __shared__ float src_scale[TMM];
+  __shared__ int dst_row[TMM];
+  int e, r0, r1;
+  if (!find_block(off, nexp, blockIdx.x, TMM, &e, &r0, &r1)) return;
+  const int tid = threadIdx.x, wv = tid >> 6, lane = tid & 63, r16 = lane & 15, g = lane >> 4;
+  if (tid < TMM) {
+    const int sp = r0 + tid;
+    if (sp < r1) {
+      const int pid = sorted[sp];
+      src_row[tid] = GLU ? pid / top : sp;
+      src_scale[tid] = GLU ? wts[pid] : 1.f;
+      dst_row[tid] = GLU ? sp : pid;
+    } else {
+      src_row[tid] = -1;
+      src_scale[tid] = 0.f;
+      dst_row[tid] = -1;
+    }
+  }
+  __syncthreads();
+  const int col = blockIdx.y * 64 + wv * 16 + r16;
+  const bool col_ok = col < N;
+  const __bf16* we = w + (int64_t)e * (GLU ? 2 : 1) * N * K;
+  const __bf16* wg = we + (int64_t)(col_ok ? col : 0) * K;
+  const __bf16* wu = we + (int64_t)(N + (col_ok ? col : 0)) * K;
+  bm_f32x4 acc[MS], acc2[GLU ? MS : 1];
+#pragma unroll
+  for (int m = 0; m < MS; m++) {
+    acc[m] = bm_f32x4{0.f, 0.f, 0.f, 0.f};
+    if (GLU) acc2[m] = bm_f32x4{0.f, 0.f, 0.f, 0.f};
+  }
+  const bm_bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+  for (int k0 = 0; k0 < K; k0 += TKK) {
+    for (int c = tid; c < TMM * 8; c += 256) {
+      const int r = c >> 3, kc = (c & 7) * 8;
+      const int sr = src_row[r];
+      bm_bf16x8 v = zero8;
+      if (sr >= 0 && k0 + kc < K) {
+        v = *(const bm_bf16x8*)(x + (int64_t)sr * K + k0 + kc);
+        if (GLU) {
+          const float sc = src_scale[r];
+#pragma unroll
+          for (int i = 0; i < 8; i++) v[i] = (__bf16)((float)v[i] * sc);
+        }
+      }
+      *(bm_bf16x8*)(as + r * AP + kc) = v;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int ks = 0; ks < 2; ks++) {
+      const int kk = k0 + ks * 32 + 8 * g;
+      const bool ok = col_ok && kk < K;
+      const bm_bf16x8 b = ok ? *(const bm_bf16x8*)(wg + kk) : zero8;
+      bm_bf16x8 b2 = zero8;
+      if (GLU && ok) b2 = *(const bm_bf16x8*)(wu + kk);
+#pragma unroll
+      for (int m = 0; m < MS; m++) {
+        const bm_bf16x8 a = *(const bm_bf16x8*)(as + (m * 16 + r16) * AP + ks * 32 + 8 * g);
+        acc[m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc[m], 0, 0, 0);
+        if (GLU) acc2[m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b2, acc2[m], 0, 0, 0);
+      }
+    }
+    __syncthreads();
+  }
+  if (!col_ok) return;
+#pragma unroll
+  for (int m = 0; m < MS; m++) {
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      const int dr = dst_row[m * 16 + 4 * g + i];
+      if (dr < 0) continue;
+      if (GLU) {
+        const float gt = fminf((float)(__bf16)acc[m][i], limit);
+        const float u = fminf(fmaxf((float)(__bf16)acc2[m][i], -limit), limit);
+        y[(int64_t)dr * N + col] = (__bf16)(gt / (1.0f + expf(-alpha * gt)) * (u + 1.0f));
+      } else {
+        outp[(int64_t)dr * N + col] = acc[m][i];
+      }
+    }
+  }
+}
+
 }  // namespace
 
 void moe_route(const float* z, int T, int E, int top, int32_t* idx, float* w, hipStream_t st) {
@@ -232,7 +331,14 @@ void moe_glu(bool bf16, const void* h, const int32_t* off, const int32_t* sorted
              const void* w_gu, void* y, int P, int E, int ff, int W, float limit, float alpha, hipStream_t st) {
   if (P <= 0) return;
   const dim3 grid((P + TM - 1) / TM + E, (ff + TN - 1) / TN);
-  if (bf16)
+  if (bf16 && W % 8 == 0) {
+    if (P / E >= 64)
+      moe_gemm_mfma_k<128, true><<<dim3((P + 127) / 128 + E, (ff + 63) / 64), 256, 0, st>>>(
+          (const __bf16*)h, off, sorted, wts, top, (const __bf16*)w_gu, (__bf16*)y, nullptr, E, ff, W, limit, alpha);
+    else
+      moe_gemm_mfma_k<32, true><<<dim3((P + 31) / 32 + E, (ff + 63) / 64), 256, 0, st>>>(
+          (const __bf16*)h, off, sorted, wts, top, (const __bf16*)w_gu, (__bf16*)y, nullptr, E, ff, W, limit, alpha);
+  } else if (bf16)
     moe_gemm_k<__bf16, true><<<grid, 256, 0, st>>>((const __bf16*)h, off, sorted, wts, top, (const __bf16*)w_gu,
                                                    (__bf16*)y, nullptr, E, ff, W, limit, alpha);
   else
@@ -244,7 +350,14 @@ void moe_down(bool bf16, const void* y, const int32_t* off, const int32_t* sorte
               int P, int E, int ff, int W, hipStream_t st) {
   if (P <= 0) return;
   const dim3 grid((P + TM - 1) / TM + E, (W + TN - 1) / TN);
-  if (bf16)
+  if (bf16 && ff % 8 == 0) {
+    if (P / E >= 64)
+      moe_gemm_mfma_k<128, false><<<dim3((P + 127) / 128 + E, (W + 63) / 64), 256, 0, st>>>(
+          (const __bf16*)y, off, sorted, nullptr, 1, (const __bf16*)w_down, nullptr, out, E, W, ff, 0.f, 0.f);
+    else
+      moe_gemm_mfma_k<32, false><<<dim3((P + 31) / 32 + E, (W + 63) / 64), 256, 0, st>>>(
+          (const __bf16*)y, off, sorted, nullptr, 1, (const __bf16*)w_down, nullptr, out, E, W, ff, 0.f, 0.f);
+  } else if (bf16)
     moe_gemm_k<__bf16, false><<<grid, 256, 0, st>>>((const __bf16*)y, off, sorted, nullptr, 1, (const __bf16*)w_down,
                                                     nullptr, out, E, W, ff, 0.f, 0.f);
   else

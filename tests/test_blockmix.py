@@ -570,3 +570,28 @@ def test_trace_replay_program(tmp_path, dev):
     assert rel_err(rd(2), wa[[99]]) < TOL[torch.float32]
     assert rel_err(rd(3), wb[[1]]) < TOL[torch.float32]
     assert rel_err(rd(4), wb[[65]]) < TOL[torch.float32]
+
+
+@pytest.mark.parametrize("T,E,top,Wd,ff", [(300, 4, 2, 72, 40), (20, 6, 3, 64, 48), (5, 3, 1, 136, 24)])
+def test_experts_bf16(dev, T, E, top, Wd, ff):
+    """16-bit experts (matrix cores on the GPU: row blocks of 128 and of 32, widths that are no multiple of the
+    k step or of the column tile) against the f64 form on the same rounded weights"""
+    from ipex_llm_amd.ops import blockmix as BM
+    g = torch.Generator().manual_seed(T)
+    h = torch.randn(T, Wd, generator=g).bfloat16()
+    z = torch.randn(T, E, generator=g)
+    idx, w = BM.moe_route(z.to(dev), top)
+    Wt = {}
+    for e in range(E):
+        Wt[f"e{e}.gate"] = (torch.randn(ff, Wd, generator=g) * Wd ** -0.5).bfloat16()
+        Wt[f"e{e}.up"] = (torch.randn(ff, Wd, generator=g) * Wd ** -0.5).bfloat16()
+        Wt[f"e{e}.down"] = (torch.randn(Wd, ff, generator=g) * ff ** -0.5).bfloat16()
+    w_gu = torch.stack([torch.cat([Wt[f"e{e}.gate"], Wt[f"e{e}.up"]]) for e in range(E)])
+    w_down = torch.stack([Wt[f"e{e}.down"] for e in range(E)])
+    got = BM.moe_experts(h.to(dev), idx, w, w_gu.to(dev), w_down.to(dev), 1.5, 1.702).cpu().double()
+    W64 = {k: v.double() for k, v in Wt.items()}
+    want = torch.zeros(T, Wd, dtype=F64)
+    for t in range(T):
+        for j in range(top):
+            want[t] += O.expert(W64, f"e{int(idx[t, j])}.", float(w[t, j]) * h[t].double(), 1.5)
+    assert (got - want).abs().max() < 0.03 * float(want.abs().max())
