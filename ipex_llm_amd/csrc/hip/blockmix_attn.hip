@@ -370,6 +370,189 @@ __global__ void __launch_bounds__(128) talk_attn_combine_k(const float* __restri
   }
 }
 
+// ------------------------------------------------------------------ long portions on the matrix cores (bf16 rows)
+// One workgroup per 16 consecutive query tokens of one sequence's portion, all H = 4 HW heads; wave w owns heads
+// w HW .. w HW + HW - 1 (their query fragments, split into bf16 hi + lo halves, and their output accumulators stay in
+// registers).  Per tile of 16 keys: keys row-major and values transposed into LDS; scores as 16x16x32 MFMAs
+// (D[key][token]); mixing over the heads and the causal mask by one thread per (token, key); online softmax by one
+// thread per (head, token) row, weights written as bf16 hi + lo; weighted sums as 16x16x16 MFMAs (D[token][column]).
+typedef short bm_s16x4 __attribute__((ext_vector_type(4)));
+constexpr int PF_KT = 16, PF_SP = PF_KT + 4, PF_PP = PF_KT + 4, PF_VP = PF_KT + 8;
+
+__host__ __device__ __forceinline__ int pf_lds_bytes(int H, int G, int d) {
+  const int Gd = G * d;
+  return 4 * (round4(H * H) + H * 16 * PF_SP + 2 * round4(H * 16)) + 2 * (PF_KT * (Gd + 8) + Gd * PF_VP + 2 * H * 16 * PF_PP);
+}
+
+template <int D16, int HW>
+__global__ void __launch_bounds__(256) talk_prefill_k(const float* __restrict__ q, const __bf16* __restrict__ rows, int bs,
+                                                     const int32_t* __restrict__ bt, const int64_t* __restrict__ pos,
+                                                     int t0, int n, float scale, const float* __restrict__ talk,
+                                                     const __bf16* __restrict__ gate, int64_t g_st,
+                                                     __bf16* __restrict__ out, int G) {
+  constexpr int H = 4 * HW, d = 16 * D16, KS = D16 / 2;
+  extern __shared__ float lds[];
+  const int tid = threadIdx.x, wv = tid >> 6, lane = tid & 63, r16 = lane & 15, gq = lane >> 4;
+  const int Gd = G * d, REP = H / G, KP = Gd + 8;
+  float* tk = lds;
+  float* S = tk + round4(H * H);
+  float* corr = S + H * 16 * PF_SP;
+  float* linv = corr + round4(H * 16);
+  __bf16* Kt = (__bf16*)(linv + round4(H * 16));
+  __bf16* Vt = Kt + PF_KT * KP;
+  __bf16* Ph = Vt + Gd * PF_VP;
+  __bf16* Pl = Ph + H * 16 * PF_PP;
+
+  const int tq0 = t0 + 16 * blockIdx.x;                       // first token of this tile
+  const int nq = t0 + n - tq0 < 16 ? t0 + n - tq0 : 16;       // valid tokens
+  const int64_t p0 = pos[tq0];                                // consecutive positions p0 .. p0 + nq - 1
+  const int64_t nkeys = p0 + nq;
+  for (int i = tid; i < H * H; i += 256) tk[i] = talk ? talk[i] : ((i / H) == (i % H) ? 1.f : 0.f);
+
+  // query fragments: lane (token r16, k part gq) of every owned head
+  bm_bf16x8 qh[HW][KS], ql[HW][KS];
+#pragma unroll
+  for (int hh = 0; hh < HW; hh++) {
+    const int h = wv * HW + hh;
+#pragma unroll
+    for (int ks = 0; ks < KS; ks++) {
+      const float* src = q + ((int64_t)(tq0 + (r16 < nq ? r16 : 0)) * H + h) * d + 32 * ks + 8 * gq;
+#pragma unroll
+      for (int e = 0; e < 8; e++) {
+        const float v = r16 < nq ? src[e] : 0.f;
+        const __bf16 hi = (__bf16)v;
+        qh[hh][ks][e] = hi;
+        ql[hh][ks][e] = (__bf16)(v - (float)hi);
+      }
+    }
+  }
+  bm_f32x4 acc[HW][D16];
+#pragma unroll
+  for (int hh = 0; hh < HW; hh++)
+#pragma unroll
+    for (int nt = 0; nt < D16; nt++) acc[hh][nt] = bm_f32x4{0.f, 0.f, 0.f, 0.f};
+  float m_run = -INFINITY, l_run = 0.f;                       // of row tid = (head tid / 16, token tid % 16)
+  const int pieces = Gd / 8;
+  const bm_bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+
+  for (int64_t j0 = 0; j0 < nkeys; j0 += PF_KT) {
+    const int nv = (int)(nkeys - j0 < PF_KT ? nkeys - j0 : PF_KT);
+    // ---- keys row-major, values transposed; rows past nv are zero
+    for (int i = tid; i < PF_KT * pieces * 2; i += 256) {
+      const int j = i / (2 * pieces), c = i - j * 2 * pieces;
+      bm_bf16x8 v = zero8;
+      if (j < nv) {
+        const int64_t kp = j0 + j;
+        const int64_t row = (int64_t)bt[kp / bs] * bs + kp % bs;
+        v = *(const bm_bf16x8*)(rows + row * 2 * Gd + c * 8);
+      }
+      if (c < pieces) {
+        *(bm_bf16x8*)(Kt + j * KP + c * 8) = v;
+      } else {
+        __bf16* dst = Vt + (int64_t)(c - pieces) * 8 * PF_VP + j;
+#pragma unroll
+        for (int e = 0; e < 8; e++) dst[e * PF_VP] = v[e];
+      }
+    }
+    __syncthreads();
+    // ---- scores: D[key 4 gq + i][token r16] of every owned head
+#pragma unroll
+    for (int hh = 0; hh < HW; hh++) {
+      const int h = wv * HW + hh, g = h / REP;
+      const __bf16* ka = Kt + r16 * KP + g * d + 8 * gq;
+      bm_f32x4 a4 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int ks = 0; ks < KS; ks++) {
+        const bm_bf16x8 a = *(const bm_bf16x8*)(ka + 32 * ks);
+        a4 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, qh[hh][ks], a4, 0, 0, 0);
+        a4 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, ql[hh][ks], a4, 0, 0, 0);
+      }
+      *(float4*)(S + (h * 16 + r16) * PF_SP + 4 * gq) = make_float4(a4[0] * scale, a4[1] * scale, a4[2] * scale, a4[3] * scale);
+    }
+    __syncthreads();
+    // ---- mixing over the heads + causal mask: thread (token tid / 16, key tid % 16)
+    {
+      const int t = tid >> 4, j = tid & 15;
+      const bool vis = t < nq && j < nv && j0 + j <= p0 + t;
+      float sv[H];
+#pragma unroll
+      for (int g = 0; g < H; g++) sv[g] = S[(g * 16 + t) * PF_SP + j];
+#pragma unroll
+      for (int h = 0; h < H; h++) {
+        float v = 0.f;
+#pragma unroll
+        for (int g = 0; g < H; g++) v += tk[h * H + g] * sv[g];
+        S[(h * 16 + t) * PF_SP + j] = vis ? v : -INFINITY;
+      }
+    }
+    __syncthreads();
+    // ---- online softmax: thread tid < 16 H owns row (head tid / 16, token tid % 16)
+    if (tid < H * 16) {
+      float sv[PF_KT];
+#pragma unroll
+      for (int c = 0; c < PF_KT / 4; c++) {
+        const float4 v = *(const float4*)(S + tid * PF_SP + 4 * c);
+        sv[4 * c] = v.x; sv[4 * c + 1] = v.y; sv[4 * c + 2] = v.z; sv[4 * c + 3] = v.w;
+      }
+      float mt = m_run;
+#pragma unroll
+      for (int j = 0; j < PF_KT; j++) mt = fmaxf(mt, sv[j]);
+      const float c = mt == -INFINITY ? 1.f : expf(m_run - mt);
+      float ls = 0.f;
+#pragma unroll
+      for (int j = 0; j < PF_KT; j++) {
+        const float pj = sv[j] == -INFINITY ? 0.f : expf(sv[j] - mt);
+        ls += pj;
+        const __bf16 hi = (__bf16)pj;
+        Ph[tid * PF_PP + j] = hi;
+        Pl[tid * PF_PP + j] = (__bf16)(pj - (float)hi);
+      }
+      l_run = l_run * c + ls;
+      m_run = mt;
+      corr[tid] = c;
+    }
+    __syncthreads();
+    // ---- weighted sums: D[token 4 gq + i][column r16] of every owned head and column tile
+#pragma unroll
+    for (int hh = 0; hh < HW; hh++) {
+      const int h = wv * HW + hh, g = h / REP;
+      const float4 c4 = *(const float4*)(corr + h * 16 + 4 * gq);
+      const bm_s16x4 ah = *(const bm_s16x4*)(Ph + (h * 16 + r16) * PF_PP + 4 * gq);
+      const bm_s16x4 al = *(const bm_s16x4*)(Pl + (h * 16 + r16) * PF_PP + 4 * gq);
+#pragma unroll
+      for (int nt = 0; nt < D16; nt++) {
+        bm_f32x4 a = acc[hh][nt];
+        a[0] *= c4.x; a[1] *= c4.y; a[2] *= c4.z; a[3] *= c4.w;
+        const bm_s16x4 b = *(const bm_s16x4*)(Vt + (g * d + nt * 16 + r16) * PF_VP + 4 * gq);
+        a = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(ah, b, a, 0, 0, 0);
+        a = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(al, b, a, 0, 0, 0);
+        acc[hh][nt] = a;
+      }
+    }
+    __syncthreads();
+  }
+  if (tid < H * 16) linv[tid] = 1.0f / l_run;
+  __syncthreads();
+#pragma unroll
+  for (int hh = 0; hh < HW; hh++) {
+    const int h = wv * HW + hh;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      const int t = 4 * gq + i;
+      if (t >= nq) continue;
+      const float li = linv[h * 16 + t];
+      const int64_t tq = tq0 + t;
+#pragma unroll
+      for (int nt = 0; nt < D16; nt++) {
+        const int o = h * d + nt * 16 + r16;
+        float v = acc[hh][nt][i] * li;
+        if (gate) v *= 1.0f / (1.0f + expf(-(float)gate[tq * g_st + o]));
+        out[tq * (int64_t)H * d + o] = (__bf16)v;
+      }
+    }
+  }
+}
+
 // ------------------------------------------------------------------ softmax step of the library-product path
 // one block per token: rows t H .. t H + H - 1 of sc [nt H, L].  Pass A mixes the H raw scores of every key
 // column (scaled) in place; pass B is the masked softmax of every row, a wave per row in turn.
@@ -517,6 +700,39 @@ void talk_attention(bool bf16, const float* q, const void* rows, int bs, const i
     else
       talk_attn_combine_k<float><<<dim3(T, H), 128, 0, st>>>(part, (const float*)gate, g_st, (float*)out, nsplit, H, d);
   }
+}
+
+bool talk_prefill_fits(int H, int G, int d) {
+  return (H == 4 || H == 8 || H == 16) && (d == 64 || d == 128) && G >= 1 && H % G == 0 &&
+         pf_lds_bytes(H, G, d) <= 150 * 1024;
+}
+
+template <int D16, int HW>
+static void launch_prefill(const float* q, const void* rows, int bs, const int32_t* bt, const int64_t* pos, int t0, int n,
+                           float scale, const float* talk, const void* gate, int64_t g_st, void* out, int G,
+                           hipStream_t st) {
+  const int H = 4 * HW, d = 16 * D16;
+  const int lds = pf_lds_bytes(H, G, d);
+  static int granted = 0;                             // dynamic LDS past 64 KB is granted per kernel
+  if (lds > granted) {
+    hipFuncSetAttribute((const void*)talk_prefill_k<D16, HW>, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+    granted = lds;
+  }
+  talk_prefill_k<D16, HW><<<(n + 15) / 16, 256, lds, st>>>(q, (const __bf16*)rows, bs, bt, pos, t0, n, scale, talk,
+                                                          (const __bf16*)gate, g_st, (__bf16*)out, G);
+}
+
+void talk_prefill(const float* q, const void* rows, int bs, const int32_t* bt, const int64_t* pos, int t0, int n,
+                  float scale, const float* talk, const void* gate, int64_t g_st, void* out, int H, int G, int d,
+                  hipStream_t st) {
+  if (n <= 0 || !talk_prefill_fits(H, G, d)) return;
+#define BM_PF(D16, HW) launch_prefill<D16, HW>(q, rows, bs, bt, pos, t0, n, scale, talk, gate, g_st, out, G, st)
+  if (d == 64) {
+    if (H == 4) BM_PF(4, 1); else if (H == 8) BM_PF(4, 2); else BM_PF(4, 4);
+  } else {
+    if (H == 4) BM_PF(8, 1); else if (H == 8) BM_PF(8, 2); else BM_PF(8, 4);
+  }
+#undef BM_PF
 }
 
 void talk_softmax(bool bf16, float* sc, const int64_t* pos, int H, float scale, const float* talk, int64_t nt, int L,

@@ -241,6 +241,44 @@ Tensor bm_talk_attention(const Tensor& q, const Tensor& rows, const Tensor& bloc
   return out;
 }
 
+int64_t bm_talk_prefill_fits(int64_t H, int64_t G, int64_t d) {
+  return illm::bm::talk_prefill_fits((int)H, (int)G, (int)d) ? 1 : 0;
+}
+
+void bm_talk_prefill(const Tensor& q, const Tensor& rows, const Tensor& table_row, const Tensor& pos, int64_t t0,
+                     int64_t n, double scale, const c10::optional<Tensor>& talk, const c10::optional<Tensor>& gate,
+                     int64_t G, Tensor& out) {
+  c10::DeviceGuard g(q.device());
+  TORCH_CHECK(q.is_cuda() && q.dim() == 3 && q.scalar_type() == at::kFloat && q.is_contiguous(),
+              "bm_talk_prefill: q f32 [T, H, d] contiguous");
+  const int64_t T = q.size(0), H = q.size(1), d = q.size(2);
+  TORCH_CHECK(illm::bm::talk_prefill_fits((int)H, (int)G, (int)d), "bm_talk_prefill: sizes outside the kernel's set");
+  TORCH_CHECK(t0 >= 0 && n >= 1 && t0 + n <= T, "bm_talk_prefill: portion outside the step");
+  TORCH_CHECK(rows.is_cuda() && rows.dim() == 3 && rows.scalar_type() == at::kBFloat16 && rows.is_contiguous() &&
+                  rows.size(2) == 2 * G * d && rows.size(1) % 64 == 0,
+              "bm_talk_prefill: rows bf16 [blocks, bs (multiple of 64), 2 G d]");
+  TORCH_CHECK(table_row.is_cuda() && table_row.scalar_type() == at::kInt && table_row.dim() == 1 &&
+                  table_row.is_contiguous(),
+              "bm_talk_prefill: block table row int32 [W]");
+  check_idx(pos, at::kLong, T, "bm_talk_prefill: pos int64 [T]");
+  const float* tp = talk_ptr(talk, H, "bm_talk_prefill: talk f32 [H, H]");
+  const void* gp = nullptr;
+  int64_t gst = 0;
+  if (gate.has_value() && gate->defined()) {
+    TORCH_CHECK(gate->is_cuda() && gate->dim() == 2 && gate->size(0) == T && gate->size(1) == H * d &&
+                    gate->scalar_type() == at::kBFloat16 && gate->stride(1) == 1,
+                "bm_talk_prefill: gate bf16 [T, H d]");
+    gp = gate->data_ptr();
+    gst = gate->stride(0);
+  }
+  TORCH_CHECK(out.is_cuda() && out.scalar_type() == at::kBFloat16 && out.is_contiguous() && out.dim() == 2 &&
+                  out.size(0) == T && out.size(1) == H * d,
+              "bm_talk_prefill: out bf16 [T, H d]");
+  illm::bm::talk_prefill(q.data_ptr<float>(), rows.data_ptr(), (int)rows.size(1), table_row.data_ptr<int32_t>(),
+                         pos.data_ptr<int64_t>(), (int)t0, (int)n, (float)scale, tp, gp, gst, out.data_ptr(), (int)H,
+                         (int)G, (int)d, stream());
+}
+
 std::tuple<Tensor, Tensor> bm_talk_softmax(Tensor& sc, const Tensor& pos, int64_t H, double scale,
                                            const c10::optional<Tensor>& talk, bool act_f32) {
   c10::DeviceGuard g(sc.device());
@@ -326,6 +364,9 @@ TORCH_LIBRARY_FRAGMENT(ipex_llm_amd, m) {
   m.def("bm_talk_attention_fits(bool bf16, int H, int G, int d) -> int");
   m.def("bm_talk_attention(Tensor q, Tensor rows, Tensor block_tables, Tensor seq_of, Tensor pos, float scale, "
         "Tensor? talk, Tensor? gate, int G, int max_ctx, bool act_f32) -> Tensor");
+  m.def("bm_talk_prefill_fits(int H, int G, int d) -> int");
+  m.def("bm_talk_prefill(Tensor q, Tensor rows, Tensor table_row, Tensor pos, int t0, int n, float scale, Tensor? talk, "
+        "Tensor? gate, int G, Tensor(a!) out) -> ()");
   m.def("bm_talk_softmax(Tensor(a!) scores, Tensor pos, int H, float scale, Tensor? talk, bool act_f32) -> "
         "(Tensor, Tensor)");
   m.def("bm_moe_route(Tensor z, int top) -> (Tensor, Tensor)");
@@ -335,6 +376,7 @@ TORCH_LIBRARY_FRAGMENT(ipex_llm_amd, m) {
 
 TORCH_LIBRARY_IMPL(ipex_llm_amd, CompositeExplicitAutograd, m) {
   m.impl("bm_talk_attention_fits", &bm_talk_attention_fits);
+  m.impl("bm_talk_prefill_fits", &bm_talk_prefill_fits);
 }
 
 TORCH_LIBRARY_IMPL(ipex_llm_amd, CUDA, m) {
@@ -347,6 +389,7 @@ TORCH_LIBRARY_IMPL(ipex_llm_amd, CUDA, m) {
   m.impl("bm_side_gate", &bm_side_gate);
   m.impl("bm_qk_norm_rope_store", &bm_qk_norm_rope_store);
   m.impl("bm_talk_attention", &bm_talk_attention);
+  m.impl("bm_talk_prefill", &bm_talk_prefill);
   m.impl("bm_talk_softmax", &bm_talk_softmax);
   m.impl("bm_moe_route", &bm_moe_route);
   m.impl("bm_moe_experts", &bm_moe_experts);

@@ -144,7 +144,11 @@ def qk_norm_rope_store(q: torch.Tensor, k: torch.Tensor, q_norm: Optional[torch.
     return qf.contiguous()
 
 
-# portions of at least this many tokens take the library-product path on the GPU
+# GPU paths by portion length.  Decoded tokens and short portions: the one-pass kernel, a workgroup per token.
+# 16-bit portions of at least MFMA_MIN_Q tokens, head sizes 64 / 128 and 4 / 8 / 16 heads: the matrix-core kernel,
+# a workgroup per 16 tokens.  Other portions of at least GEMM_MIN_Q tokens (and every portion of sizes the one-pass
+# kernel cannot hold): library products with the fused mixing softmax between them.
+MFMA_MIN_Q = int(__import__("os").environ.get("ILLM_TALK_MFMA_MIN", "32"))
 GEMM_MIN_Q = int(__import__("os").environ.get("ILLM_TALK_GEMM_MIN", "128"))
 GEMM_Q_BLOCK = int(__import__("os").environ.get("ILLM_TALK_GEMM_BLOCK", "512"))
 
@@ -234,15 +238,18 @@ def _talk_attention_gpu(q, rows, block_tables, seq_of, pos, scale, talk, gate, G
     T, H, d = q.shape
     f32 = out_dtype == torch.float32
     fits = _ops().bm_talk_attention_fits(not f32, H, G, d) > 0
-    min_q = GEMM_MIN_Q if fits else 1
-    big = [b for b, n in enumerate(q_lens) if n >= min_q]
-    if not big:
+    mfma = not f32 and MFMA_MIN_Q > 0 and _ops().bm_talk_prefill_fits(H, G, d) > 0
+    min_q = (min(MFMA_MIN_Q, GEMM_MIN_Q) if mfma else GEMM_MIN_Q) if fits else 1
+    if all(n < min_q for n in q_lens):
         return _ops().bm_talk_attention(q.contiguous(), rows, block_tables, seq_of, pos, scale, talk, gate, G,
                                         max(ctx_lens), f32)
+    q = q.contiguous()
     out = torch.empty(T, H * d, dtype=out_dtype, device=q.device)
     small, small_ctx, t0 = [], 1, 0
     for b, (n, L) in enumerate(zip(q_lens, ctx_lens)):
-        if n >= min_q:
+        if n >= min_q and mfma:
+            _ops().bm_talk_prefill(q, rows, block_tables[b], pos, t0, n, scale, talk, gate, G, out)
+        elif n >= min_q:
             o = _talk_attention_gemm(q[t0:t0 + n], rows, block_tables[b], pos[t0:t0 + n], scale, talk, G, L, n)
             o = o.view(n, H * d)
             if gate is not None:

@@ -275,35 +275,38 @@ def test_causal_edge(dev, edge):
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("H,G,d", [(8, 2, 64), (6, 3, 40), (5, 5, 16)])
-def test_long_portion_library_path_equals_flash(H, G, d, dtype):
-    """portions past the threshold take library products with the fused mixing softmax between them;
-    the same rows through the one-pass kernel give the same result"""
+@pytest.mark.parametrize("H,G,d", [(8, 2, 64), (16, 4, 128), (4, 4, 64), (8, 1, 128), (6, 3, 40), (5, 5, 16)])
+def test_long_portion_paths_agree(H, G, d, dtype):
+    """portions past the thresholds take the matrix-core kernel (16-bit, its sizes) or library products with the
+    fused mixing softmax between them; the same rows through the one-pass kernel give the same result.  The
+    portion starts inside a page, ends inside a 16-token tile and shares the step with a decoded token."""
     if not torch.cuda.is_available():
         pytest.skip("no GPU")
     from ipex_llm_amd.ops import blockmix as BM
     dev = torch.device("cuda")
     g = torch.Generator().manual_seed(d)
-    L, n = 700, 640                                   # the portion starts 60 tokens into the sequence
+    L, n = 700, 633                                   # the portion starts 67 tokens into the sequence
     k, v = torch.randn(L, G, d, generator=g).to(dtype), torch.randn(L, G, d, generator=g).to(dtype)
-    q = torch.randn(n, H, d, generator=g)
+    q = torch.randn(n + 1, H, d, generator=g)
     talk = torch.eye(H) + 0.3 * torch.randn(H, H, generator=g)
-    gate = torch.randn(n, H * d, generator=g).to(dtype)
+    gate = torch.randn(n + 1, H * d, generator=g).to(dtype)
     rows, bt = paged_rows(k, v, dev, dtype, seed=d)
-    positions = list(range(L - n, L))
-    args = (q.to(dev), rows, bt, torch.zeros(n, dtype=torch.int32, device=dev), torch.tensor(positions, device=dev), 0.25,
-            talk.to(dev), gate.to(dev), G, [n], [L], dtype)
-    lib = BM.talk_attention(*args).cpu().double()
-    old = BM.GEMM_MIN_Q
-    BM.GEMM_MIN_Q = 1 << 30
-    try:
-        flash = BM.talk_attention(*args).cpu().double()
-    finally:
-        BM.GEMM_MIN_Q = old
-    want = plain_mixed_attention(q.double(), k.double(), v.double(), talk.double(), 0.25, positions).reshape(n, H * d) * \
+    bt = torch.cat([bt, bt])                          # a second sequence over the same pages brings one token
+    positions = list(range(L - n, L)) + [L - 5]
+    seq_of = torch.tensor([0] * n + [1], dtype=torch.int32, device=dev)
+    args = (q.to(dev), rows, bt, seq_of, torch.tensor(positions, device=dev), 0.25, talk.to(dev), gate.to(dev), G,
+            [n, 1], [L, L - 4], dtype)
+    want = plain_mixed_attention(q.double(), k.double(), v.double(), talk.double(), 0.25, positions).reshape(n + 1, H * d) * \
         torch.sigmoid(gate.double())
     tol = 2e-5 if dtype == torch.float32 else 2e-2
-    assert (lib - want).abs().max() < tol and (flash - want).abs().max() < tol
+    old = BM.GEMM_MIN_Q, BM.MFMA_MIN_Q
+    try:
+        for gemm_min, mfma_min in (old, (128, 0), (1 << 30, 0)):
+            BM.GEMM_MIN_Q, BM.MFMA_MIN_Q = gemm_min, mfma_min
+            got = BM.talk_attention(*args).cpu().double()
+            assert (got - want).abs().max() < tol, (gemm_min, mfma_min)
+    finally:
+        BM.GEMM_MIN_Q, BM.MFMA_MIN_Q = old
 
 
 def test_qk_norm_rotation_and_rows(dev):
