@@ -371,43 +371,42 @@ __global__ void __launch_bounds__(128) talk_attn_combine_k(const float* __restri
 }
 
 // ------------------------------------------------------------------ long portions on the matrix cores (bf16 rows)
-// One workgroup per 16 consecutive query tokens of one sequence's portion, all H = 4 HW heads; wave w owns heads
+// One workgroup of NW waves per 16 consecutive query tokens of one sequence's portion, all H = NW HW heads; wave w owns heads
 // w HW .. w HW + HW - 1 (their query fragments, split into bf16 hi + lo halves, and their output accumulators stay in
-// registers).  Per tile of 16 keys: keys row-major and values transposed into LDS; scores as 16x16x32 MFMAs
-// (D[key][token]); mixing over the heads and the causal mask by one thread per (token, key); online softmax by one
-// thread per (head, token) row, weights written as bf16 hi + lo; weighted sums as 16x16x16 MFMAs (D[token][column]).
+// registers).  Per tile of 16 keys: the cache rows as they are into LDS; scores as 16x16x32 MFMAs (D[key][token]);
+// mixing over the heads as one small MFMA product per token (matrix and scores as bf16 hi + lo halves) with the
+// causal mask; online softmax by one thread per (head, token) row, weights written as bf16 hi + lo; weighted sums as 16x16x16 MFMAs (D[token][column]) whose value
+// operand a lane gathers from four rows (16 lanes read 32 contiguous bytes, the four row groups fall into other banks).
 typedef short bm_s16x4 __attribute__((ext_vector_type(4)));
-constexpr int PF_KT = 16, PF_SP = PF_KT + 4, PF_PP = PF_KT + 4, PF_VP = PF_KT + 8;
+constexpr int PF_KT = 16, PF_SP = PF_KT + 4, PF_PP = PF_KT + 4;
 
 __host__ __device__ __forceinline__ int pf_lds_bytes(int H, int G, int d) {
   const int Gd = G * d;
-  return 4 * (round4(H * H) + H * 16 * PF_SP + 2 * round4(H * 16)) + 2 * (PF_KT * (Gd + 8) + Gd * PF_VP + 2 * H * 16 * PF_PP);
+  return 4 * (round4(H * H) + H * 16 * PF_SP + 2 * round4(H * 16)) + 2 * (PF_KT * (2 * Gd + 8) + 2 * H * 16 * PF_PP);
 }
 
-template <int D16, int HW>
-__global__ void __launch_bounds__(256) talk_prefill_k(const float* __restrict__ q, const __bf16* __restrict__ rows, int bs,
+template <int D16, int HW, int NW>
+__global__ void __launch_bounds__(64 * NW) talk_prefill_k(const float* __restrict__ q, const __bf16* __restrict__ rows, int bs,
                                                      const int32_t* __restrict__ bt, const int64_t* __restrict__ pos,
                                                      int t0, int n, float scale, const float* __restrict__ talk,
                                                      const __bf16* __restrict__ gate, int64_t g_st,
                                                      __bf16* __restrict__ out, int G) {
-  constexpr int H = 4 * HW, d = 16 * D16, KS = D16 / 2;
+  constexpr int H = NW * HW, d = 16 * D16, KS = D16 / 2, NT = 64 * NW, TPW = 16 / NW;
   extern __shared__ float lds[];
   const int tid = threadIdx.x, wv = tid >> 6, lane = tid & 63, r16 = lane & 15, gq = lane >> 4;
-  const int Gd = G * d, REP = H / G, KP = Gd + 8;
+  const int Gd = G * d, REP = H / G, KP = 2 * Gd + 8;
   float* tk = lds;
   float* S = tk + round4(H * H);
   float* corr = S + H * 16 * PF_SP;
   float* linv = corr + round4(H * 16);
   __bf16* Kt = (__bf16*)(linv + round4(H * 16));
-  __bf16* Vt = Kt + PF_KT * KP;
-  __bf16* Ph = Vt + Gd * PF_VP;
+  __bf16* Ph = Kt + PF_KT * KP;
   __bf16* Pl = Ph + H * 16 * PF_PP;
 
-  const int tq0 = t0 + 16 * blockIdx.x;                       // first token of this tile
+  const int tq0 = t0 + 16 * (gridDim.x - 1 - blockIdx.x);     // first token of this tile; the longest tiles start first
   const int nq = t0 + n - tq0 < 16 ? t0 + n - tq0 : 16;       // valid tokens
   const int64_t p0 = pos[tq0];                                // consecutive positions p0 .. p0 + nq - 1
   const int64_t nkeys = p0 + nq;
-  for (int i = tid; i < H * H; i += 256) tk[i] = talk ? talk[i] : ((i / H) == (i % H) ? 1.f : 0.f);
 
   // query fragments: lane (token r16, k part gq) of every owned head
   bm_bf16x8 qh[HW][KS], ql[HW][KS];
@@ -426,6 +425,17 @@ __global__ void __launch_bounds__(256) talk_prefill_k(const float* __restrict__ 
       }
     }
   }
+  bm_s16x4 th = {0, 0, 0, 0}, tl = {0, 0, 0, 0};               // mixing matrix: lane (head r16, g part gq)
+  if (talk) {
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+      const int g = 4 * gq + e;
+      const float v = (r16 < H && g < H) ? talk[r16 * H + g] : 0.f;
+      const __bf16 hi = (__bf16)v;
+      th[e] = __builtin_bit_cast(short, hi);
+      tl[e] = __builtin_bit_cast(short, (__bf16)(v - (float)hi));
+    }
+  }
   bm_f32x4 acc[HW][D16];
 #pragma unroll
   for (int hh = 0; hh < HW; hh++)
@@ -435,26 +445,35 @@ __global__ void __launch_bounds__(256) talk_prefill_k(const float* __restrict__ 
   const int pieces = Gd / 8;
   const bm_bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
 
+  // a tile's 16 rows lie in one page, one after the other: 16-byte pieces tid, tid + 256, ... of that run.  The next
+  // tile's pieces are requested before the current tile's arithmetic and land in LDS after it.
+  constexpr int kMaxNL = 2048 / NT;                           // 2 G d <= 1024
+  const int npiece = PF_KT * pieces * 2;
+  bm_bf16x8 pre[kMaxNL];
+  auto request = [&](int64_t j0) {
+    const int nvr = (int)(nkeys - j0 < PF_KT ? nkeys - j0 : PF_KT);
+    const __bf16* src = rows + ((int64_t)bt[j0 / bs] * bs + j0 % bs) * 2 * Gd;
+#pragma unroll
+    for (int it = 0; it < kMaxNL; it++) {
+      const int i = tid + NT * it;
+      pre[it] = zero8;
+      if (i < npiece && i / (2 * pieces) < nvr) pre[it] = *(const bm_bf16x8*)(src + (int64_t)i * 8);
+    }
+  };
+  request(0);
   for (int64_t j0 = 0; j0 < nkeys; j0 += PF_KT) {
     const int nv = (int)(nkeys - j0 < PF_KT ? nkeys - j0 : PF_KT);
-    // ---- keys row-major, values transposed; rows past nv are zero
-    for (int i = tid; i < PF_KT * pieces * 2; i += 256) {
-      const int j = i / (2 * pieces), c = i - j * 2 * pieces;
-      bm_bf16x8 v = zero8;
-      if (j < nv) {
-        const int64_t kp = j0 + j;
-        const int64_t row = (int64_t)bt[kp / bs] * bs + kp % bs;
-        v = *(const bm_bf16x8*)(rows + row * 2 * Gd + c * 8);
-      }
-      if (c < pieces) {
-        *(bm_bf16x8*)(Kt + j * KP + c * 8) = v;
-      } else {
-        __bf16* dst = Vt + (int64_t)(c - pieces) * 8 * PF_VP + j;
+    // ---- the tile's rows [keys | values]; rows past nv are zero
 #pragma unroll
-        for (int e = 0; e < 8; e++) dst[e * PF_VP] = v[e];
+    for (int it = 0; it < kMaxNL; it++) {
+      const int i = tid + NT * it;
+      if (i < npiece) {
+        const int j = i / (2 * pieces), c = i - j * 2 * pieces;
+        *(bm_bf16x8*)(Kt + j * KP + c * 8) = pre[it];
       }
     }
     __syncthreads();
+    if (j0 + PF_KT < nkeys) request(j0 + PF_KT);
     // ---- scores: D[key 4 gq + i][token r16] of every owned head
 #pragma unroll
     for (int hh = 0; hh < HW; hh++) {
@@ -470,19 +489,33 @@ __global__ void __launch_bounds__(256) talk_prefill_k(const float* __restrict__ 
       *(float4*)(S + (h * 16 + r16) * PF_SP + 4 * gq) = make_float4(a4[0] * scale, a4[1] * scale, a4[2] * scale, a4[3] * scale);
     }
     __syncthreads();
-    // ---- mixing over the heads + causal mask: thread (token tid / 16, key tid % 16)
-    {
-      const int t = tid >> 4, j = tid & 15;
-      const bool vis = t < nq && j < nv && j0 + j <= p0 + t;
-      float sv[H];
+    // ---- mixing over the heads + causal mask: wave w takes 16 / NW tokens; per token one 16 x 16 x 16
+    // product D[head][key] = T[head][g] S[g][key], T and S as bf16 hi + lo halves (hi hi + hi lo + lo hi)
 #pragma unroll
-      for (int g = 0; g < H; g++) sv[g] = S[(g * 16 + t) * PF_SP + j];
+    for (int tt = 0; tt < TPW; tt++) {
+      const int t = wv * TPW + tt;
+      const bool vis = t < nq && r16 < nv && j0 + r16 <= p0 + t;
+      if (talk) {
+        bm_s16x4 bh, bl;
 #pragma unroll
-      for (int h = 0; h < H; h++) {
-        float v = 0.f;
+        for (int e = 0; e < 4; e++) {
+          const int g = 4 * gq + e;
+          const float v = g < H ? S[(g * 16 + t) * PF_SP + r16] : 0.f;
+          const __bf16 hi = (__bf16)v;
+          bh[e] = __builtin_bit_cast(short, hi);
+          bl[e] = __builtin_bit_cast(short, (__bf16)(v - (float)hi));
+        }
+        bm_f32x4 m4 = {0.f, 0.f, 0.f, 0.f};
+        m4 = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(th, bh, m4, 0, 0, 0);
+        m4 = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(th, bl, m4, 0, 0, 0);
+        m4 = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(tl, bh, m4, 0, 0, 0);
 #pragma unroll
-        for (int g = 0; g < H; g++) v += tk[h * H + g] * sv[g];
-        S[(h * 16 + t) * PF_SP + j] = vis ? v : -INFINITY;
+        for (int i = 0; i < 4; i++)
+          if (4 * gq + i < H) S[((4 * gq + i) * 16 + t) * PF_SP + r16] = vis ? m4[i] : -INFINITY;
+      } else if (!vis) {
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+          if (4 * gq + i < H) S[((4 * gq + i) * 16 + t) * PF_SP + r16] = -INFINITY;
       }
     }
     __syncthreads();
@@ -497,15 +530,23 @@ __global__ void __launch_bounds__(256) talk_prefill_k(const float* __restrict__ 
       float mt = m_run;
 #pragma unroll
       for (int j = 0; j < PF_KT; j++) mt = fmaxf(mt, sv[j]);
-      const float c = mt == -INFINITY ? 1.f : expf(m_run - mt);
+      const float c = mt == -INFINITY ? 1.f : __expf(m_run - mt);
       float ls = 0.f;
 #pragma unroll
-      for (int j = 0; j < PF_KT; j++) {
-        const float pj = sv[j] == -INFINITY ? 0.f : expf(sv[j] - mt);
-        ls += pj;
-        const __bf16 hi = (__bf16)pj;
-        Ph[tid * PF_PP + j] = hi;
-        Pl[tid * PF_PP + j] = (__bf16)(pj - (float)hi);
+      for (int c4i = 0; c4i < PF_KT / 4; c4i++) {
+        bm_s16x4 hi4, lo4;
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+          const float sj = sv[4 * c4i + e];
+          const float pj = sj == -INFINITY ? 0.f : __expf(sj - mt);
+          ls += pj;
+          const __bf16 hi = (__bf16)pj;
+          const __bf16 lo = (__bf16)(pj - (float)hi);
+          hi4[e] = __builtin_bit_cast(short, hi);
+          lo4[e] = __builtin_bit_cast(short, lo);
+        }
+        *(bm_s16x4*)(Ph + tid * PF_PP + 4 * c4i) = hi4;
+        *(bm_s16x4*)(Pl + tid * PF_PP + 4 * c4i) = lo4;
       }
       l_run = l_run * c + ls;
       m_run = mt;
@@ -513,20 +554,52 @@ __global__ void __launch_bounds__(256) talk_prefill_k(const float* __restrict__ 
     }
     __syncthreads();
     // ---- weighted sums: D[token 4 gq + i][column r16] of every owned head and column tile
+    {
+      float4 c4[HW];
+      bm_s16x4 ah[HW], al[HW];
 #pragma unroll
-    for (int hh = 0; hh < HW; hh++) {
-      const int h = wv * HW + hh, g = h / REP;
-      const float4 c4 = *(const float4*)(corr + h * 16 + 4 * gq);
-      const bm_s16x4 ah = *(const bm_s16x4*)(Ph + (h * 16 + r16) * PF_PP + 4 * gq);
-      const bm_s16x4 al = *(const bm_s16x4*)(Pl + (h * 16 + r16) * PF_PP + 4 * gq);
+      for (int hh = 0; hh < HW; hh++) {
+        const int h = wv * HW + hh;
+        c4[hh] = *(const float4*)(corr + h * 16 + 4 * gq);
+        ah[hh] = *(const bm_s16x4*)(Ph + (h * 16 + r16) * PF_PP + 4 * gq);
+        al[hh] = *(const bm_s16x4*)(Pl + (h * 16 + r16) * PF_PP + 4 * gq);
+      }
+      bool moved = false;
+#pragma unroll
+      for (int hh = 0; hh < HW; hh++)
+        moved |= c4[hh].x != 1.f || c4[hh].y != 1.f || c4[hh].z != 1.f || c4[hh].w != 1.f;
+      if (__any(moved)) {                             // some running maximum of this wave's rows grew
+#pragma unroll
+        for (int hh = 0; hh < HW; hh++)
+#pragma unroll
+          for (int nt = 0; nt < D16; nt++) {
+            acc[hh][nt][0] *= c4[hh].x;
+            acc[hh][nt][1] *= c4[hh].y;
+            acc[hh][nt][2] *= c4[hh].z;
+            acc[hh][nt][3] *= c4[hh].w;
+          }
+      }
+      const short* vbase = (const short*)Kt + (4 * gq) * KP + Gd + r16;
 #pragma unroll
       for (int nt = 0; nt < D16; nt++) {
-        bm_f32x4 a = acc[hh][nt];
-        a[0] *= c4.x; a[1] *= c4.y; a[2] *= c4.z; a[3] *= c4.w;
-        const bm_s16x4 b = *(const bm_s16x4*)(Vt + (g * d + nt * 16 + r16) * PF_VP + 4 * gq);
-        a = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(ah, b, a, 0, 0, 0);
-        a = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(al, b, a, 0, 0, 0);
-        acc[hh][nt] = a;
+        bm_s16x4 b = {0, 0, 0, 0};
+        int gprev = -1;
+#pragma unroll
+        for (int hh = 0; hh < HW; hh++) {
+          const int g = (wv * HW + hh) / REP;
+          if (g != gprev) {                           // keys 4 gq .. 4 gq + 3 at column nt 16 + r16 of value head g
+            const short* vb = vbase + g * d + nt * 16;
+            b[0] = vb[0];
+            b[1] = vb[KP];
+            b[2] = vb[2 * KP];
+            b[3] = vb[3 * KP];
+            gprev = g;
+          }
+          bm_f32x4 a = acc[hh][nt];
+          a = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(ah[hh], b, a, 0, 0, 0);
+          a = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(al[hh], b, a, 0, 0, 0);
+          acc[hh][nt] = a;
+        }
       }
     }
     __syncthreads();
@@ -703,22 +776,22 @@ void talk_attention(bool bf16, const float* q, const void* rows, int bs, const i
 }
 
 bool talk_prefill_fits(int H, int G, int d) {
-  return (H == 4 || H == 8 || H == 16) && (d == 64 || d == 128) && G >= 1 && H % G == 0 &&
+  return (H == 4 || H == 8 || H == 16) && (d == 64 || d == 128) && G >= 1 && H % G == 0 && G * d <= 512 &&
          pf_lds_bytes(H, G, d) <= 150 * 1024;
 }
 
-template <int D16, int HW>
+template <int D16, int HW, int NW>
 static void launch_prefill(const float* q, const void* rows, int bs, const int32_t* bt, const int64_t* pos, int t0, int n,
                            float scale, const float* talk, const void* gate, int64_t g_st, void* out, int G,
                            hipStream_t st) {
-  const int H = 4 * HW, d = 16 * D16;
+  const int H = NW * HW, d = 16 * D16;
   const int lds = pf_lds_bytes(H, G, d);
   static int granted = 0;                             // dynamic LDS past 64 KB is granted per kernel
   if (lds > granted) {
-    hipFuncSetAttribute((const void*)talk_prefill_k<D16, HW>, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+    hipFuncSetAttribute((const void*)talk_prefill_k<D16, HW, NW>, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
     granted = lds;
   }
-  talk_prefill_k<D16, HW><<<(n + 15) / 16, 256, lds, st>>>(q, (const __bf16*)rows, bs, bt, pos, t0, n, scale, talk,
+  talk_prefill_k<D16, HW, NW><<<(n + 15) / 16, 64 * NW, lds, st>>>(q, (const __bf16*)rows, bs, bt, pos, t0, n, scale, talk,
                                                           (const __bf16*)gate, g_st, (__bf16*)out, G);
 }
 
@@ -726,11 +799,11 @@ void talk_prefill(const float* q, const void* rows, int bs, const int32_t* bt, c
                   float scale, const float* talk, const void* gate, int64_t g_st, void* out, int H, int G, int d,
                   hipStream_t st) {
   if (n <= 0 || !talk_prefill_fits(H, G, d)) return;
-#define BM_PF(D16, HW) launch_prefill<D16, HW>(q, rows, bs, bt, pos, t0, n, scale, talk, gate, g_st, out, G, st)
+#define BM_PF(D16, HW, NW) launch_prefill<D16, HW, NW>(q, rows, bs, bt, pos, t0, n, scale, talk, gate, g_st, out, G, st)
   if (d == 64) {
-    if (H == 4) BM_PF(4, 1); else if (H == 8) BM_PF(4, 2); else BM_PF(4, 4);
+    if (H == 4) BM_PF(4, 1, 4); else if (H == 8) BM_PF(4, 2, 4); else BM_PF(4, 2, 8);
   } else {
-    if (H == 4) BM_PF(8, 1); else if (H == 8) BM_PF(8, 2); else BM_PF(8, 4);
+    if (H == 4) BM_PF(8, 1, 4); else if (H == 8) BM_PF(8, 1, 8); else BM_PF(8, 2, 8);
   }
 #undef BM_PF
 }
