@@ -200,7 +200,8 @@ def paged_rows(k, v, dev, dtype, bs=64, spare=3, seed=0):
     return rows.to(dev, dtype), perm.to(torch.int32)[None].to(dev)
 
 
-@pytest.mark.parametrize("H,G,d", [(4, 2, 16), (8, 2, 64), (6, 6, 8), (5, 1, 24), (16, 4, 32), (3, 3, 128)])
+@pytest.mark.parametrize("H,G,d", [(4, 2, 16), (8, 2, 64), (6, 6, 8), (5, 1, 24), (16, 4, 32), (3, 3, 128), (12, 1, 20),
+                                   (2, 2, 12)])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_mixed_score_attention_op(dev, H, G, d, dtype):
     """decoded tokens and short portions over shuffled pages, keys past 200, with and without the mixing matrix"""
@@ -275,7 +276,8 @@ def test_causal_edge(dev, edge):
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("H,G,d", [(8, 2, 64), (16, 4, 128), (4, 4, 64), (8, 1, 128), (6, 3, 40), (5, 5, 16)])
+@pytest.mark.parametrize("H,G,d", [(8, 2, 64), (16, 4, 128), (4, 4, 64), (8, 1, 128), (16, 2, 64), (4, 1, 128), (6, 3, 40),
+                                   (5, 5, 16), (12, 1, 20), (3, 3, 12)])
 def test_long_portion_paths_agree(H, G, d, dtype):
     """portions past the thresholds take the matrix-core kernel (16-bit, its sizes) or library products with the
     fused mixing softmax between them; the same rows through the one-pass kernel give the same result.  The
@@ -381,7 +383,22 @@ LAYER_CASES = [
     ([O.attn_layer(heads=6, kv_heads=1, dim=16, dims=8, mlp=O.moe(6, 2, 16, 1.0, 24, 3.0))], dict(width=40, taps=4, side=5)),
     ([O.attn_layer(heads=2, kv_heads=1, dim=40, mlp=O.moe(4, 4, 8, 2.0))], dict(width=16, taps=3, side=3)),
     ([O.attn_layer(heads=1, kv_heads=1, dim=8, mlp=O.moe(2, 1, 8, 0.5, 8, 0.5))], dict(width=8, taps=1, side=1)),
+    # head sizes that are no multiple of 8 and more than 8 query heads per key / value head: no one-pass kernel
+    ([O.attn_layer(heads=5, kv_heads=5, dim=12, dims=6, mlp=O.moe(3, 2, 12, 2.0, 20, 1.0))], dict(width=20, taps=3, side=2)),
+    ([O.attn_layer(heads=12, kv_heads=1, dim=20, scaling=YARN, mlp=O.dense(36))], dict(width=36, taps=2, side=0)),
 ]
+
+
+@pytest.mark.parametrize("case", [2, 5, 6])
+def test_one_layer_models_bf16(dev, case):
+    """16-bit serving of odd sizes: decoded tokens and portions through whatever path the sizes allow"""
+    layers, kw = LAYER_CASES[case]
+    cfg = O.config(layers, **kw)
+    W = O.random_weights(cfg, case)
+    seed = max(range(40), key=lambda s: O.router_margin(cfg, W, O.random_tokens(cfg, 80, s)))
+    toks = O.random_tokens(cfg, 80, seed)
+    got = replay(engine(cfg, W, dev, torch.bfloat16), {"a": toks}, [[("a", 70)], [("a", 3)]] + [[("a", 1)]] * 7)["a"]
+    assert rel_err(got, O.forward(cfg, W, toks)) < TOL[torch.bfloat16]
 
 
 @pytest.mark.parametrize("case", range(len(LAYER_CASES)))
@@ -575,7 +592,7 @@ def test_trace_replay_program(tmp_path, dev):
     assert rel_err(rd(4), wb[[65]]) < TOL[torch.float32]
 
 
-@pytest.mark.parametrize("T,E,top,Wd,ff", [(300, 4, 2, 72, 40), (20, 6, 3, 64, 48), (5, 3, 1, 136, 24)])
+@pytest.mark.parametrize("T,E,top,Wd,ff", [(300, 4, 2, 72, 40), (20, 6, 3, 64, 48), (5, 3, 1, 136, 24), (9, 3, 2, 20, 12)])
 def test_experts_bf16(dev, T, E, top, Wd, ff):
     """16-bit experts (matrix cores on the GPU: row blocks of 128 and of 32, widths that are no multiple of the
     k step or of the column tile) against the f64 form on the same rounded weights"""
