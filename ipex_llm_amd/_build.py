@@ -96,8 +96,10 @@ def _cmd(src: str, obj: str):
 # partial libraries: the translation units one model kind needs, linked alone
 TARGETS = {
     # hybrid decoders: sequence-mixing kernels + their bindings + the serving scheduler
+    # (+ the streaming skinny-GEMM kernel their decode-size projections share with the dense decoders)
     "seqmix": ["hip/seqmix.hip", "hip/blockmix_elem.hip", "hip/blockmix_attn.hip", "hip/blockmix_moe.hip",
-               "torch/ops_seqmix.cpp", "torch/ops_blockmix.cpp", "runtime/scheduler.cpp"],
+               "hip/dense_gemv.hip", "torch/ops_seqmix.cpp", "torch/ops_blockmix.cpp", "torch/ops_dense.cpp",
+               "runtime/scheduler.cpp"],
 }
 
 
@@ -120,6 +122,8 @@ def needs_build(target=None) -> bool:
     if not os.path.exists(lib):
         return True
     newest = max([os.path.getmtime(s) for s in sources(target)] + [_headers_mtime()])
+    if target:                                  # the list of units a partial library links is in this file
+        newest = max(newest, os.path.getmtime(os.path.abspath(__file__)))
     return os.path.getmtime(lib) < newest
 
 
@@ -154,7 +158,8 @@ def build(verbose: bool = False, jobs: int | None = None, force: bool = False, t
             return src
         with cf.ThreadPoolExecutor(jobs) as ex:
             list(ex.map(run, todo))
-    need_link = todo or not os.path.exists(LIB) or any(os.path.getmtime(o) > os.path.getmtime(LIB) for o in objs)
+    need_link = todo or not os.path.exists(LIB) or any(os.path.getmtime(o) > os.path.getmtime(LIB) for o in objs) or \
+        (target is not None and os.path.getmtime(os.path.abspath(__file__)) > os.path.getmtime(LIB))
     if need_link:
         _, _, tlib = _torch_paths()
         cmd = [HIPCC, "-shared", "-fPIC", f"--offload-arch={ARCH}", *objs, "-o", LIB + ".tmp",

@@ -732,7 +732,7 @@ int talk_attention_splits(bool bf16, int T, int H, int G, int d, int max_ctx) {
   const int tiles = (max_ctx + kt - 1) / kt;
   int ns = 1;
   // fill the chip (256 CUs, a few workgroups each), at least 4 tiles per split
-  while (ns < 64 && (int64_t)T * ns < 512 && tiles / (ns * 2) >= 4) ns *= 2;
+  while (ns < 64 && (int64_t)T * ns < 1024 && tiles / (ns * 2) >= 2) ns *= 2;
   return ns;
 }
 

@@ -275,14 +275,14 @@ class GroupedAttention(nn.Module):
     def forward(self, xa, pos, slots, meta: AttnMeta, cache, li: int, eps: float):
         s = self.s
         T, H, G, d = xa.shape[0], s.heads, s.kv_heads, s.dim
-        y = F.linear(xa, self.w_in)
+        y = BM.linear(xa, self.w_in)
         q = y[:, :H * d].view(T, H, d)
         k = y[:, H * d:(H + G) * d].view(T, G, d)
         gate = y[:, (H + G) * d:] if s.out_gate else None
         qf = BM.qk_norm_rope_store(q, k, self.q_norm, self.k_norm, eps, self.table, pos, slots, cache.rows[li])
         o = BM.talk_attention(qf, cache.rows[li], meta.block_tables, meta.seq_of, pos, s.scale, self.talk, gate, G,
                               meta.q_lens_host, meta.seq_lens_host, xa.dtype)
-        return F.linear(o, self.w_o)
+        return BM.linear(o, self.w_o)
 
 
 class ReluSqFF(nn.Module):
@@ -292,7 +292,7 @@ class ReluSqFF(nn.Module):
         self.w_down = nn.Parameter(w_down, requires_grad=False)
 
     def forward(self, xa, x32=None):
-        return F.linear(BM.relu_sq(F.linear(xa, self.w_up)), self.w_down), None
+        return BM.linear(BM.relu_sq(BM.linear(xa, self.w_up)), self.w_down), None
 
 
 class SigmoidMoE(nn.Module):
@@ -314,7 +314,7 @@ class SigmoidMoE(nn.Module):
         y = BM.moe_experts(xa, idx, wts, self.w_gu, self.w_down, s.expert.limit, s.expert.alpha)
         ys = None
         if self.shared_gu is not None:
-            ys = F.linear(BM.glu_clamp(F.linear(xa, self.shared_gu), s.shared.limit, s.shared.alpha), self.shared_down)
+            ys = BM.linear(BM.glu_clamp(BM.linear(xa, self.shared_gu), s.shared.limit, s.shared.alpha), self.shared_down)
         return y, ys
 
 
@@ -330,8 +330,8 @@ class TokenSide(nn.Module):
         self.offset = offset
 
     def forward(self, x, xa, ids, table, eps: float, act):
-        g = BM.side_gate(F.linear(xa, self.w_gate), table, ids, self.offset)
-        return BM.add_rms_norm_(x, F.linear(g, self.w_proj), self.norm, eps, act)
+        g = BM.side_gate(BM.linear(xa, self.w_gate), table, ids, self.offset)
+        return BM.add_rms_norm_(x, BM.linear(g, self.w_proj), self.norm, eps, act)
 
 
 class HybridLayer(nn.Module):
@@ -496,4 +496,4 @@ class HybridCausalLM(nn.Module):
             xn = BM.rms_norm_rows(x, self.norm, s.norm_eps, act)[1]
         if return_hidden:
             return xn
-        return F.linear(xn, self.lm_head).float()
+        return BM.linear(xn, self.lm_head).float()

@@ -23,12 +23,23 @@ import torch.nn.functional as F
 
 from .seqmix import native, _mm_f32
 
-__all__ = ["rms_norm_rows", "canon_conv", "qk_norm_rope_store", "talk_attention", "relu_sq", "glu_clamp",
+__all__ = ["linear", "rms_norm_rows", "canon_conv", "qk_norm_rope_store", "talk_attention", "relu_sq", "glu_clamp",
            "residual_add_scaled_", "side_gate", "add_rms_norm_", "moe_route", "moe_experts"]
 
 
 def _ops():
     return torch.ops.ipex_llm_amd
+
+
+# ------------------------------------------------------------------ projections
+def linear(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
+    """``x W^T`` for rows ``x`` [T, K] and ``w`` [N, K]: decode-size steps (at most 16 rows, 16-bit) stream the
+    weight once through the skinny-GEMM kernel the dense decoders use (csrc/hip/dense_gemv.hip), everything
+    else is a library GEMM."""
+    if x.is_cuda and x.dim() == 2 and x.shape[0] <= 16 and x.dtype == torch.bfloat16 and w.dtype == x.dtype and \
+            x.shape[1] % 8 == 0 and w.is_contiguous() and native(x):
+        return _ops().dense_linear(x, w, None)
+    return F.linear(x, w)
 
 
 # ------------------------------------------------------------------ norms
