@@ -184,8 +184,36 @@ __global__ void __launch_bounds__(256) talk_attn_k(const float* __restrict__ q, 
   const bool pv_on = JS > 1 ? tid < JS * Gd : true;
   __syncthreads();
 
+  // MF: a tile's rows lie in one page, one after the other (KT divides the page size), so the tile is one run of
+  // 16-byte pieces; the next tile's pieces are requested before the current tile's arithmetic
+  constexpr int kMaxPre = MF ? 8 : 1;
+  uint4 pre[kMaxPre];
+  const int npiece = KT * (row_w / 4);
+  auto request = [&](int64_t j0) {
+    const int nvr = (int)(k_hi - j0 < KT ? k_hi - j0 : KT);
+    const uint4* src = (const uint4*)((const uint32_t*)rows + ((int64_t)bt[j0 / bs] * bs + j0 % bs) * row_w);
+#pragma unroll
+    for (int it = 0; it < kMaxPre; it++) {
+      const int i = tid + 256 * it;
+      pre[it] = make_uint4(0u, 0u, 0u, 0u);
+      if (i < npiece && i / (row_w / 4) < nvr) pre[it] = src[i];
+    }
+  };
+  if (MF && k_lo < k_hi) request(k_lo);
   for (int64_t j0 = k_lo; j0 < k_hi; j0 += KT) {
     const int nv = (int)(k_hi - j0 < KT ? k_hi - j0 : KT);
+    if (MF) {
+#pragma unroll
+      for (int it = 0; it < kMaxPre; it++) {
+        const int i = tid + 256 * it;
+        if (i < npiece && i / (row_w / 4) < nv) {
+          const int j = i / (row_w / 4), c = i - j * (row_w / 4);
+          *(uint4*)(tile + j * pitch + c * 4) = pre[it];
+        }
+      }
+      __syncthreads();
+      if (j0 + KT < k_hi) request(j0 + KT);
+    } else {
     // ---- tile load: 16-byte pieces of the nv rows
     {
       const int pieces = row_w / 4;                 // row_w is a multiple of 4 words (d % 8 == 0)
@@ -195,17 +223,14 @@ __global__ void __launch_bounds__(256) talk_attn_k(const float* __restrict__ q, 
         const int64_t row = (int64_t)bt[kp / bs] * bs + kp % bs;
         const uint4 v = *(const uint4*)((const uint32_t*)rows + row * row_w + c * 4);
         uint32_t* dst = tile + j * pitch + c * 4;
-        if (MF) {
-          *(uint4*)dst = v;
-        } else {
-          dst[0] = v.x;
-          dst[1] = v.y;
-          dst[2] = v.z;
-          dst[3] = v.w;
-        }
+        dst[0] = v.x;
+        dst[1] = v.y;
+        dst[2] = v.z;
+        dst[3] = v.w;
       }
     }
     __syncthreads();
+    }
     // ---- scores
     if (MF) {
       const int r16 = lane & 15, gq = lane >> 4;
@@ -718,6 +743,7 @@ int talk_attention_plan(bool bf16, int H, int G, int d, int* kt) {
   const int pitch = mf ? 2 * G * d / per + 4 : ((2 * G * d / per) | 1);
   for (int KT = 64; KT >= (mf ? 16 : 8); KT >>= 1) {
     const int64_t bytes = (int64_t)lds_floats(H, G, d, KT) * 4 + (int64_t)KT * pitch * 4;
+    if (mf && (int64_t)KT * (2 * G * d / per) / 4 > 8 * 256) continue;       // the prefetch registers hold 8 pieces
     if (bytes <= 64 * 1024) {
       *kt = KT;
       return (int)bytes;
