@@ -266,34 +266,57 @@ __global__ void __launch_bounds__(256) moe_gemm_mfma_k(const __bf16* __restrict_
     if (GLU) acc2[m] = bm_f32x4{0.f, 0.f, 0.f, 0.f};
   }
   const bm_bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
-  for (int k0 = 0; k0 < K; k0 += TKK) {
-    for (int c = tid; c < TMM * 8; c += 256) {
+  // the next k step's operands (gathered row pieces, this wave's weight fragments) are requested before the
+  // current step's products and used after them
+  constexpr int NA = TMM * 8 / 256;
+  bm_bf16x8 pa[NA], pb[2], pb2[2];
+  auto request = [&](int k0) {
+#pragma unroll
+    for (int it = 0; it < NA; it++) {
+      const int c = tid + 256 * it;
       const int r = c >> 3, kc = (c & 7) * 8;
       const int sr = src_row[r];
-      bm_bf16x8 v = zero8;
-      if (sr >= 0 && k0 + kc < K) {
-        v = *(const bm_bf16x8*)(x + (int64_t)sr * K + k0 + kc);
-        if (GLU) {
-          const float sc = src_scale[r];
-#pragma unroll
-          for (int i = 0; i < 8; i++) v[i] = (__bf16)((float)v[i] * sc);
-        }
-      }
-      *(bm_bf16x8*)(as + r * AP + kc) = v;
+      pa[it] = zero8;
+      if (sr >= 0 && k0 + kc < K) pa[it] = *(const bm_bf16x8*)(x + (int64_t)sr * K + k0 + kc);
     }
-    __syncthreads();
 #pragma unroll
     for (int ks = 0; ks < 2; ks++) {
       const int kk = k0 + ks * 32 + 8 * g;
       const bool ok = col_ok && kk < K;
-      const bm_bf16x8 b = ok ? *(const bm_bf16x8*)(wg + kk) : zero8;
-      bm_bf16x8 b2 = zero8;
-      if (GLU && ok) b2 = *(const bm_bf16x8*)(wu + kk);
+      pb[ks] = ok ? *(const bm_bf16x8*)(wg + kk) : zero8;
+      pb2[ks] = zero8;
+      if (GLU && ok) pb2[ks] = *(const bm_bf16x8*)(wu + kk);
+    }
+  };
+  request(0);
+  for (int k0 = 0; k0 < K; k0 += TKK) {
+#pragma unroll
+    for (int it = 0; it < NA; it++) {
+      const int c = tid + 256 * it;
+      const int r = c >> 3, kc = (c & 7) * 8;
+      bm_bf16x8 v = pa[it];
+      if (GLU) {
+        const float sc = src_scale[r];
+#pragma unroll
+        for (int i = 0; i < 8; i++) v[i] = (__bf16)((float)v[i] * sc);
+      }
+      *(bm_bf16x8*)(as + r * AP + kc) = v;
+    }
+    bm_bf16x8 b[2], b2[2];
+#pragma unroll
+    for (int ks = 0; ks < 2; ks++) {
+      b[ks] = pb[ks];
+      b2[ks] = pb2[ks];
+    }
+    __syncthreads();
+    if (k0 + TKK < K) request(k0 + TKK);
+#pragma unroll
+    for (int ks = 0; ks < 2; ks++) {
 #pragma unroll
       for (int m = 0; m < MS; m++) {
         const bm_bf16x8 a = *(const bm_bf16x8*)(as + (m * 16 + r16) * AP + ks * 32 + 8 * g);
-        acc[m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc[m], 0, 0, 0);
-        if (GLU) acc2[m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b2, acc2[m], 0, 0, 0);
+        acc[m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b[ks], acc[m], 0, 0, 0);
+        if (GLU) acc2[m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b2[ks], acc2[m], 0, 0, 0);
       }
     }
     __syncthreads();
