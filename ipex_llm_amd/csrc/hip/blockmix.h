@@ -25,6 +25,11 @@ void residual_add_scaled(bool bf16, float* x, const void* y1, const float* s1, c
 void canon_conv(bool bf16, const float* h, const float* w, int taps, float* state, const int32_t* cu,
                 const int32_t* seq_of, const int32_t* slots, const int64_t* pos, void* out, int T, int B, int W,
                 hipStream_t st);
+// rms_norm_rows + canon_conv in one launch (h f32, ha: h in the activation type (bf16 only), out = h + conv(h));
+// single: every sequence brings exactly one token (the state is advanced by the same launch)
+void norm_canon(bool bf16, const float* x, const void* g, int ng, float eps, const float* w, int taps, float* state,
+                const int32_t* cu, const int32_t* seq_of, const int32_t* slots, const int64_t* pos, float* h, void* ha,
+                void* out, int T, int B, int W, bool single, hipStream_t st);
 void relu_sq(bool bf16, const void* y, void* out, int64_t n, hipStream_t st);
 void glu_clamp(bool bf16, const void* gu, void* out, int64_t T, int64_t I, float limit, float alpha, hipStream_t st);
 // out = gelu_tanh(z) * table[ids, offset : offset + n]

@@ -147,6 +147,66 @@ __global__ void __launch_bounds__(256) canon_state_k(const float* __restrict__ h
   }
 }
 
+// RMS norm + the convolution in one launch, one block per token: h_t = x_t / rms(x_t) * g and
+// out_t = h_t + sum_j w[:, j] h_(t - taps + 1 + j).  The block norms its own row and recomputes the norms of the
+// earlier rows of its portion that the taps reach (same formula and reduction order as for their own blocks);
+// what lies before the portion comes from the state.  ``single``: every sequence brings one token, so the block
+// is the only reader of its sequence's state and advances it itself; otherwise canon_state_k follows.
+constexpr int kMaxTaps = 16;
+template <typename E>
+__global__ void __launch_bounds__(256) norm_canon_k(const float* __restrict__ x, const E* __restrict__ g, int ng,
+                                                   float eps, const float* __restrict__ w, int taps,
+                                                   float* __restrict__ state, const int32_t* __restrict__ cu,
+                                                   const int32_t* __restrict__ seq_of, const int32_t* __restrict__ slots,
+                                                   const int64_t* __restrict__ pos, float* __restrict__ h,
+                                                   E* __restrict__ ha, E* __restrict__ out, int W, int single) {
+  __shared__ float red[16];
+  const int64_t t = blockIdx.x;
+  const int b = seq_of[t];
+  const int64_t t_start = cu[b];
+  const int64_t p = pos[t], p0 = p - (t - t_start);
+  const int nh = taps - 1;
+  float* st = state + (int64_t)slots[b] * nh * W;
+  float rs[kMaxTaps];
+#pragma unroll
+  for (int r = 0; r < kMaxTaps; r++) {
+    rs[r] = 0.f;
+    if (r < taps && p - r >= p0) {                  // uniform over the block
+      const float* xr = x + (t - r) * W;
+      float q = 0.f;
+      for (int c = threadIdx.x; c < W; c += blockDim.x) q += xr[c] * xr[c];
+      rs[r] = 1.0f / sqrtf(block_sum(q, red) / (float)W + eps);
+    }
+  }
+  const float g0 = ldf(g);
+  for (int c = threadIdx.x; c < W; c += blockDim.x) {
+    const float gc = ng == 1 ? g0 : ldf(g + c);
+    const float own = x[t * W + c] * rs[0] * gc;
+    float acc = own;
+    float keep[kMaxTaps];
+#pragma unroll
+    for (int r = 0; r < kMaxTaps; r++) {
+      if (r < taps) {
+        const int64_t sp = p - r;                   // the tap r positions back: weight column taps - 1 - r
+        float v = 0.f;
+        if (r == 0) v = own;
+        else if (sp >= p0) v = x[(t - r) * W + c] * rs[r] * gc;
+        else if (sp >= 0) v = st[(sp - (p0 - nh)) * W + c];
+        keep[r] = v;
+        acc += w[c * taps + (taps - 1 - r)] * v;
+      }
+    }
+    h[t * W + c] = own;
+    if (ha) stf(ha + t * W + c, own);
+    stf(out + t * W + c, acc);
+    if (single) {                                   // new state: positions p - nh + 1 .. p, oldest first
+#pragma unroll
+      for (int r = 0; r < kMaxTaps - 1; r++)
+        if (r < nh) st[(nh - 1 - r) * W + c] = keep[r];
+    }
+  }
+}
+
 template <typename E>
 __global__ void __launch_bounds__(256) relu_sq_k(const E* __restrict__ y, E* __restrict__ out, int64_t n) {
   for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) {
@@ -217,6 +277,19 @@ void canon_conv(bool bf16, const float* h, const float* w, int taps, float* stat
   if (bf16) canon_conv_k<__bf16><<<T, 256, 0, st>>>(h, w, taps, state, cu, seq_of, slots, pos, (__bf16*)out, W);
   else canon_conv_k<float><<<T, 256, 0, st>>>(h, w, taps, state, cu, seq_of, slots, pos, (float*)out, W);
   canon_state_k<<<B, 256, 0, st>>>(h, taps, state, cu, slots, pos, W);
+}
+
+void norm_canon(bool bf16, const float* x, const void* g, int ng, float eps, const float* w, int taps, float* state,
+                const int32_t* cu, const int32_t* seq_of, const int32_t* slots, const int64_t* pos, float* h, void* ha,
+                void* out, int T, int B, int W, bool single, hipStream_t st) {
+  if (T <= 0) return;
+  if (bf16)
+    norm_canon_k<__bf16><<<T, 256, 0, st>>>(x, (const __bf16*)g, ng, eps, w, taps, state, cu, seq_of, slots, pos, h,
+                                            (__bf16*)ha, (__bf16*)out, W, single ? 1 : 0);
+  else
+    norm_canon_k<float><<<T, 256, 0, st>>>(x, (const float*)g, ng, eps, w, taps, state, cu, seq_of, slots, pos, h,
+                                           nullptr, (float*)out, W, single ? 1 : 0);
+  if (!single) canon_state_k<<<B, 256, 0, st>>>(h, taps, state, cu, slots, pos, W);
 }
 
 void relu_sq(bool bf16, const void* y, void* out, int64_t n, hipStream_t st) {

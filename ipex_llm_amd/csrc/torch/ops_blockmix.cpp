@@ -119,6 +119,39 @@ Tensor bm_canon_conv(const Tensor& h, const Tensor& w, Tensor& state, const Tens
   return out;
 }
 
+std::tuple<Tensor, Tensor, Tensor> bm_norm_canon(const Tensor& x, const Tensor& g, double eps, const Tensor& w,
+                                                 Tensor& state, const Tensor& cu, const Tensor& seq_of,
+                                                 const Tensor& slots, const Tensor& pos, bool single, bool act_f32) {
+  c10::DeviceGuard gd(x.device());
+  check_f32_rows(x, "bm_norm_canon: x f32 [T, W]");
+  const int64_t T = x.size(0), W = x.size(1);
+  TORCH_CHECK(g.is_cuda() && g.is_contiguous() && (g.numel() == 1 || g.numel() == W) &&
+                  g.scalar_type() == act_type(act_f32),
+              "bm_norm_canon: norm weight [1] or [W] in the activation dtype");
+  TORCH_CHECK(w.is_cuda() && w.scalar_type() == at::kFloat && w.is_contiguous() && w.dim() == 2 && w.size(0) == W &&
+                  w.size(1) >= 2 && w.size(1) <= 16,
+              "bm_norm_canon: w f32 [W, taps], 2 <= taps <= 16");
+  const int64_t taps = w.size(1);
+  TORCH_CHECK(state.is_cuda() && state.scalar_type() == at::kFloat && state.is_contiguous() && state.dim() == 3 &&
+                  state.size(1) == taps - 1 && state.size(2) == W,
+              "bm_norm_canon: state f32 [slots, taps - 1, W]");
+  TORCH_CHECK(cu.is_cuda() && cu.scalar_type() == at::kInt && cu.is_contiguous() && cu.numel() >= 2,
+              "bm_norm_canon: cu int32 [B + 1]");
+  const int64_t B = cu.numel() - 1;
+  TORCH_CHECK(!single || B == T, "bm_norm_canon: single needs one token per sequence");
+  check_idx(seq_of, at::kInt, T, "bm_norm_canon: seq_of int32 [T]");
+  check_idx(slots, at::kInt, B, "bm_norm_canon: state slots int32 [B]");
+  check_idx(pos, at::kLong, T, "bm_norm_canon: pos int64 [T]");
+  Tensor h = at::empty({T, W}, x.options());
+  Tensor ha = act_f32 ? h : at::empty({T, W}, x.options().dtype(at::kBFloat16));
+  Tensor out = at::empty({T, W}, x.options().dtype(act_type(act_f32)));
+  illm::bm::norm_canon(!act_f32, x.data_ptr<float>(), g.data_ptr(), (int)g.numel(), (float)eps, w.data_ptr<float>(),
+                       (int)taps, state.data_ptr<float>(), cu.data_ptr<int32_t>(), seq_of.data_ptr<int32_t>(),
+                       slots.data_ptr<int32_t>(), pos.data_ptr<int64_t>(), h.data_ptr<float>(),
+                       act_f32 ? nullptr : ha.data_ptr(), out.data_ptr(), (int)T, (int)B, (int)W, single, stream());
+  return {h, ha, out};
+}
+
 Tensor bm_relu_sq(const Tensor& y) {
   c10::DeviceGuard g(y.device());
   TORCH_CHECK(y.is_cuda() && is_act(y) && y.is_contiguous(), "bm_relu_sq: contiguous bf16 / f32");
@@ -356,6 +389,8 @@ TORCH_LIBRARY_FRAGMENT(ipex_llm_amd, m) {
         "bool act_f32) -> Tensor");
   m.def("bm_canon_conv(Tensor h, Tensor w, Tensor(a!) state, Tensor cu, Tensor seq_of, Tensor slots, Tensor pos, "
         "bool act_f32) -> Tensor");
+  m.def("bm_norm_canon(Tensor x, Tensor g, float eps, Tensor w, Tensor(a!) state, Tensor cu, Tensor seq_of, Tensor slots, "
+        "Tensor pos, bool single, bool act_f32) -> (Tensor, Tensor, Tensor)");
   m.def("bm_relu_sq(Tensor y) -> Tensor");
   m.def("bm_glu_clamp(Tensor gu, float limit, float alpha) -> Tensor");
   m.def("bm_side_gate(Tensor z, Tensor table, Tensor ids, int offset) -> Tensor");
@@ -384,6 +419,7 @@ TORCH_LIBRARY_IMPL(ipex_llm_amd, CUDA, m) {
   m.impl("bm_add_rms_norm", &bm_add_rms_norm);
   m.impl("bm_residual_add_scaled", &bm_residual_add_scaled);
   m.impl("bm_canon_conv", &bm_canon_conv);
+  m.impl("bm_norm_canon", &bm_norm_canon);
   m.impl("bm_relu_sq", &bm_relu_sq);
   m.impl("bm_glu_clamp", &bm_glu_clamp);
   m.impl("bm_side_gate", &bm_side_gate);

@@ -375,14 +375,12 @@ class ParallelLayer(nn.Module):
 
     def forward(self, x, xa, ids, pos, slots, meta, cache, li: int, model):
         s, act = model.spec, model.dtype
-        h32, ha = BM.rms_norm_rows(x, self.norm1, s.norm_eps, act)
-        hm = ha
-        if self.canon is not None:
-            if self.canon.shape[1] > 1:
-                hm = BM.canon_conv(h32, self.canon, cache.state[li]["canon"], meta.cu_q, meta.seq_of, meta.state_slots,
-                                   pos, meta.q_lens_host, act)
-            else:
-                hm = (h32 * (1.0 + self.canon[:, 0])).to(act)
+        if self.canon is not None and self.canon.shape[1] > 1:
+            h32, ha, hm = BM.norm_canon(x, self.norm1, s.norm_eps, self.canon, cache.state[li]["canon"], meta.cu_q,
+                                        meta.seq_of, meta.state_slots, pos, meta.q_lens_host, act)
+        else:
+            h32, ha = BM.rms_norm_rows(x, self.norm1, s.norm_eps, act)
+            hm = ha if self.canon is None else (h32 * (1.0 + self.canon[:, 0])).to(act)
         ym = self.mixer(hm, pos, slots, meta, cache, li, s.norm_eps)
         y2, y3 = self.mlp(ha, h32) if self.mlp is not None else (None, None)
         xa = BM.residual_add_scaled_(x, ym, self.ls1, y2, y3, self.ls2, act)

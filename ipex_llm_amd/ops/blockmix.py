@@ -23,7 +23,7 @@ import torch.nn.functional as F
 
 from .seqmix import native, _mm_f32
 
-__all__ = ["linear", "rms_norm_rows", "canon_conv", "qk_norm_rope_store", "talk_attention", "relu_sq", "glu_clamp",
+__all__ = ["linear", "rms_norm_rows", "canon_conv", "norm_canon", "qk_norm_rope_store", "talk_attention", "relu_sq", "glu_clamp",
            "residual_add_scaled_", "side_gate", "add_rms_norm_", "moe_route", "moe_experts"]
 
 
@@ -115,6 +115,20 @@ def canon_conv(h: torch.Tensor, w: torch.Tensor, state: torch.Tensor, cu: torch.
         state[slots[b]] = ext[n:]
         t0 += n
     return out if act_dtype == torch.float32 else out.to(act_dtype)
+
+
+def norm_canon(x: torch.Tensor, norm_w: torch.Tensor, eps: float, w: torch.Tensor, state: torch.Tensor, cu: torch.Tensor,
+               seq_of: torch.Tensor, state_slots: torch.Tensor, pos: torch.Tensor, q_lens: List[int],
+               act_dtype: torch.dtype) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """``rms_norm_rows`` then ``canon_conv`` (one launch on the GPU; a step in which every sequence brings one
+    token also advances the state in it).  Returns the norm's result in f32 and in ``act_dtype`` and
+    ``h + conv(h)`` in ``act_dtype``."""
+    if native(x):
+        single = len(q_lens) == x.shape[0] and all(n == 1 for n in q_lens)
+        return _ops().bm_norm_canon(x.contiguous(), norm_w.reshape(-1), eps, w, state, cu, seq_of, state_slots, pos,
+                                    single, act_dtype == torch.float32)
+    h, ha = rms_norm_rows(x, norm_w, eps, act_dtype)
+    return h, ha, canon_conv(h, w, state, cu, seq_of, state_slots, pos, q_lens, act_dtype)
 
 
 # ------------------------------------------------------------------ grouped attention with mixed scores

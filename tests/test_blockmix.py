@@ -173,6 +173,39 @@ def test_canon_convolution_state(dev, taps):
     assert (torch.cat(got_b).double() - O.canon(hb.double(), w.double())).abs().max() < 1e-5
 
 
+@pytest.mark.parametrize("taps", [2, 4])
+def test_norm_and_convolution_in_one(dev, taps):
+    """the norm and the convolution as one op: mixed steps and steps in which both sequences bring one token
+    (the state then advances inside the same launch), one number and a vector as norm weight"""
+    from ipex_llm_amd.ops import blockmix as BM
+    g = torch.Generator().manual_seed(10 + taps)
+    Wd, na, nb = 21, 17, 12
+    xa_, xb_ = torch.randn(na, Wd, generator=g) * 2, torch.randn(nb, Wd, generator=g) * 2
+    w = torch.randn(Wd, taps, generator=g)
+    for nw in (torch.tensor([0.8]), 1 + 0.2 * torch.randn(Wd, generator=g)):
+        state = torch.randn(3, taps - 1, Wd, generator=g).to(dev) * 50
+        outs_a, outs_b, hs = [], [], []
+        plan = [(4, 1), (1, 1), (1, 1), (1, 3), (6, 2), (1, 1), (3, 3)]
+        ia = ib = 0
+        for ca, cb in plan:
+            x = torch.cat([xa_[ia:ia + ca], xb_[ib:ib + cb]]).to(dev)
+            cu = torch.tensor([0, ca, ca + cb], dtype=torch.int32, device=dev)
+            seq_of = torch.tensor([0] * ca + [1] * cb, dtype=torch.int32, device=dev)
+            pos = torch.tensor(list(range(ia, ia + ca)) + list(range(ib, ib + cb)), device=dev)
+            h, ha, out = BM.norm_canon(x, nw.to(dev), 1e-5, w.to(dev), state, cu, seq_of,
+                                       torch.tensor([1, 2], dtype=torch.int32, device=dev), pos, [ca, cb], torch.float32)
+            assert ha is h
+            outs_a.append(out[:ca].cpu())
+            outs_b.append(out[ca:].cpu())
+            hs.append(h[:ca].cpu())
+            ia, ib = ia + ca, ib + cb
+        assert ia == na and ib == nb
+        ha64, hb64 = O.unit_rms(xa_.double(), 1e-5) * nw.double(), O.unit_rms(xb_.double(), 1e-5) * nw.double()
+        assert (torch.cat(hs).double() - ha64).abs().max() < 1e-5
+        assert (torch.cat(outs_a).double() - O.canon(ha64, w.double())).abs().max() < 2e-5
+        assert (torch.cat(outs_b).double() - O.canon(hb64, w.double())).abs().max() < 2e-5
+
+
 def plain_mixed_attention(q, k, v, talk, scale, positions):
     """q [n, H, d] at ``positions``; k, v [L, G, d] -> [n, H, d] (f64)"""
     n, H, d = q.shape
