@@ -7,9 +7,10 @@
 //   talk_attn_k            one workgroup per (query token, key split): all H
 //                          heads of the token together, because the scores of
 //                          all heads at a key are mixed by an [H, H] matrix
-//                          before the softmax.  Per key tile: scores (f32),
-//                          mixing, causal mask, online softmax, weighted sum
-//                          of the values (f32 accumulators in registers).
+//                          before the softmax.  Per key tile: scores (f32);
+//                          mixing, causal mask and online softmax (16 lanes
+//                          per head); weighted sum of the values (f32
+//                          accumulators in registers).
 //   talk_attn_combine_k    merge of the key splits + sigmoid output gate
 //   talk_softmax_k         the scale + mixing + mask + softmax step of the
 //                          library-product path of long portions
@@ -284,35 +285,46 @@ __global__ void __launch_bounds__(256) talk_attn_k(const float* __restrict__ q, 
       }
     }
     __syncthreads();
-    // ---- mixing over the heads + mask
-    for (int it = tid; it < KT * H; it += 256) {
-      const int j = it % KT, h = it / KT;
-      float v = -INFINITY;
-      if (j < nv) {
-        v = 0.f;
-        for (int g = 0; g < H; g++) v += tk[h * H + g] * S[g * KP + j];
-      }
-      S2[h * KP + j] = v;
-    }
-    __syncthreads();
-    // ---- online softmax: a wave per head in turn; weights go to S
-    for (int h = wv; h < H; h += 4) {
-      float mt = -INFINITY;
-      for (int j = lane; j < KT; j += 64) mt = fmaxf(mt, S2[h * KP + j]);
-      mt = wave_max(mt);
-      const float mo = mrun[h], mn = fmaxf(mo, mt);
-      float ls = 0.f;
-      for (int j = lane; j < KT; j += 64) {
-        const float pj = j < nv ? expf(S2[h * KP + j] - mn) : 0.f;
-        S[h * KP + j] = pj;
-        ls += pj;
-      }
-      ls = wave_sum(ls);
-      if (lane == 0) {
-        const float c = expf(mo - mn);              // mo = -inf at the first tile: 0
-        corr[h] = c;
-        lrun[h] = lrun[h] * c + ls;
-        mrun[h] = mn;
+    // ---- mixing over the heads, mask and online softmax in one phase: 16 lanes per head (four heads per wave
+    // at a time), lane gl takes keys gl, gl + 16, ...; the weights go to S2 (S is still read by the other heads)
+    {
+      const int gl = lane & 15, hq = lane >> 4;
+      for (int h0 = wv * 4; h0 < H; h0 += 16) {
+        const int h = h0 + hq;
+        if (h < H) {
+          float sj[4];
+          float mt = -INFINITY;
+#pragma unroll
+          for (int u = 0; u < 4; u++) {
+            const int j = gl + 16 * u;
+            float v = -INFINITY;
+            if (j < nv) {
+              v = 0.f;
+              for (int g = 0; g < H; g++) v += tk[h * H + g] * S[g * KP + j];
+            }
+            sj[u] = v;
+            mt = fmaxf(mt, v);
+          }
+#pragma unroll
+          for (int o = 8; o > 0; o >>= 1) mt = fmaxf(mt, __shfl_xor(mt, o, 64));
+          const float mo = mrun[h], mn = fmaxf(mo, mt);
+          float ls = 0.f;
+#pragma unroll
+          for (int u = 0; u < 4; u++) {
+            const int j = gl + 16 * u;
+            const float pj = sj[u] == -INFINITY ? 0.f : expf(sj[u] - mn);
+            if (j < KT) S2[h * KP + j] = pj;
+            ls += pj;
+          }
+#pragma unroll
+          for (int o = 8; o > 0; o >>= 1) ls += __shfl_xor(ls, o, 64);
+          if (gl == 0) {
+            const float c = expf(mo - mn);            // mo = -inf at the first tile: 0
+            corr[h] = c;
+            lrun[h] = lrun[h] * c + ls;
+            mrun[h] = mn;
+          }
+        }
       }
     }
     __syncthreads();
@@ -329,7 +341,7 @@ __global__ void __launch_bounds__(256) talk_attn_k(const float* __restrict__ q, 
         for (int j = js; j < nv; j += JS) {
           const float v = ldf(vcol + (int64_t)j * pitch * per);
 #pragma unroll
-          for (int r = 0; r < REP; r++) acc[a][r] += S[(g * REP + r) * KP + j] * v;
+          for (int r = 0; r < REP; r++) acc[a][r] += S2[(g * REP + r) * KP + j] * v;
         }
       }
     }
