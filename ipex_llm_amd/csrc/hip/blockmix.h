@@ -53,9 +53,11 @@ void talk_attention(bool bf16, const float* q, const void* rows, int bs, const i
 // long portions of one sequence on the matrix cores (bf16 rows): tokens t0 .. t0 + n - 1 of the step at consecutive
 // positions, bt: the sequence's block table row; writes out rows t0 .. t0 + n - 1 ([T, H d] bf16)
 bool talk_prefill_fits(int H, int G, int d);
+// part: f32 scratch [n, nsplit, H, d + 2] when nsplit > 1 (talk_prefill_splits)
+int talk_prefill_splits(int n, int max_keys);
 void talk_prefill(const float* q, const void* rows, int bs, const int32_t* bt, const int64_t* pos, int t0, int n,
-                  float scale, const float* talk, const void* gate, int64_t g_st, void* out, int H, int G, int d,
-                  hipStream_t st);
+                  float scale, const float* talk, const void* gate, int64_t g_st, void* out, float* part, int nsplit,
+                  int H, int G, int d, hipStream_t st);
 // rows [R, L] of raw scores (row i = token i / H, head i % H): scaled, mixed over the heads of a token, masked by
 // pos[i / H], softmax; bf16: weights leave as hi + lo bf16 pairs (row stride L), f32 (hi == null): in place
 void talk_softmax(bool bf16, float* sc, const int64_t* pos, int H, float scale, const float* talk, int64_t nt, int L,

@@ -427,7 +427,8 @@ __global__ void __launch_bounds__(64 * NW) talk_prefill_k(const float* __restric
                                                      const int32_t* __restrict__ bt, const int64_t* __restrict__ pos,
                                                      int t0, int n, float scale, const float* __restrict__ talk,
                                                      const __bf16* __restrict__ gate, int64_t g_st,
-                                                     __bf16* __restrict__ out, int G) {
+                                                     __bf16* __restrict__ out, int G, float* __restrict__ part,
+                                                     int nsplit) {
   constexpr int H = NW * HW, d = 16 * D16, KS = D16 / 2, NT = 64 * NW, TPW = 16 / NW;
   extern __shared__ float lds[];
   const int tid = threadIdx.x, wv = tid >> 6, lane = tid & 63, r16 = lane & 15, gq = lane >> 4;
@@ -443,7 +444,10 @@ __global__ void __launch_bounds__(64 * NW) talk_prefill_k(const float* __restric
   const int tq0 = t0 + 16 * (gridDim.x - 1 - blockIdx.x);     // first token of this tile; the longest tiles start first
   const int nq = t0 + n - tq0 < 16 ? t0 + n - tq0 : 16;       // valid tokens
   const int64_t p0 = pos[tq0];                                // consecutive positions p0 .. p0 + nq - 1
-  const int64_t nkeys = p0 + nq;
+  // key splits (blockIdx.y): whole 16-key tiles of the keys the tile's last token sees; a split past them is empty
+  const int64_t tiles_total = (p0 + nq + PF_KT - 1) / PF_KT, tiles_per = (tiles_total + nsplit - 1) / nsplit;
+  const int64_t k_lo = (int64_t)blockIdx.y * tiles_per * PF_KT;
+  const int64_t nkeys = p0 + nq < k_lo + tiles_per * PF_KT ? p0 + nq : k_lo + tiles_per * PF_KT;
 
   // query fragments: lane (token r16, k part gq) of every owned head
   bm_bf16x8 qh[HW][KS], ql[HW][KS];
@@ -497,8 +501,8 @@ __global__ void __launch_bounds__(64 * NW) talk_prefill_k(const float* __restric
       if (i < npiece && i / (2 * pieces) < nvr) pre[it] = *(const bm_bf16x8*)(src + (int64_t)i * 8);
     }
   };
-  request(0);
-  for (int64_t j0 = 0; j0 < nkeys; j0 += PF_KT) {
+  if (k_lo < nkeys) request(k_lo);
+  for (int64_t j0 = k_lo; j0 < nkeys; j0 += PF_KT) {
     const int nv = (int)(nkeys - j0 < PF_KT ? nkeys - j0 : PF_KT);
     // ---- the tile's rows [keys | values]; rows past nv are zero
 #pragma unroll
@@ -640,6 +644,27 @@ __global__ void __launch_bounds__(64 * NW) talk_prefill_k(const float* __restric
       }
     }
     __syncthreads();
+  }
+  if (nsplit > 1) {
+    // unnormalised sums, running maximum and sum of every (token, head) row: merged by talk_attn_combine_k
+    if (tid < H * 16 && (tid & 15) < nq) {
+      float* pr = part + (((int64_t)(tq0 - t0 + (tid & 15)) * nsplit + blockIdx.y) * H + (tid >> 4)) * (d + 2);
+      pr[d] = m_run;
+      pr[d + 1] = l_run;
+    }
+#pragma unroll
+    for (int hh = 0; hh < HW; hh++) {
+      const int h = wv * HW + hh;
+#pragma unroll
+      for (int i = 0; i < 4; i++) {
+        const int t = 4 * gq + i;
+        if (t >= nq) continue;
+        float* pr = part + (((int64_t)(tq0 - t0 + t) * nsplit + blockIdx.y) * H + h) * (d + 2);
+#pragma unroll
+        for (int nt = 0; nt < D16; nt++) pr[nt * 16 + r16] = acc[hh][nt][i];
+      }
+    }
+    return;
   }
   if (tid < H * 16) linv[tid] = 1.0f / l_run;
   __syncthreads();
@@ -820,8 +845,8 @@ bool talk_prefill_fits(int H, int G, int d) {
 
 template <int D16, int HW, int NW>
 static void launch_prefill(const float* q, const void* rows, int bs, const int32_t* bt, const int64_t* pos, int t0, int n,
-                           float scale, const float* talk, const void* gate, int64_t g_st, void* out, int G,
-                           hipStream_t st) {
+                           float scale, const float* talk, const void* gate, int64_t g_st, void* out, int G, float* part,
+                           int nsplit, hipStream_t st) {
   const int H = NW * HW, d = 16 * D16;
   const int lds = pf_lds_bytes(H, G, d);
   static int granted = 0;                             // dynamic LDS past 64 KB is granted per kernel
@@ -829,15 +854,26 @@ static void launch_prefill(const float* q, const void* rows, int bs, const int32
     hipFuncSetAttribute((const void*)talk_prefill_k<D16, HW, NW>, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
     granted = lds;
   }
-  talk_prefill_k<D16, HW, NW><<<(n + 15) / 16, 64 * NW, lds, st>>>(q, (const __bf16*)rows, bs, bt, pos, t0, n, scale, talk,
-                                                          (const __bf16*)gate, g_st, (__bf16*)out, G);
+  talk_prefill_k<D16, HW, NW><<<dim3((n + 15) / 16, nsplit), 64 * NW, lds, st>>>(
+      q, (const __bf16*)rows, bs, bt, pos, t0, n, scale, talk, (const __bf16*)gate, g_st, (__bf16*)out, G, part, nsplit);
+  if (nsplit > 1)
+    talk_attn_combine_k<__bf16><<<dim3(n, H), 128, 0, st>>>(part, gate ? (const __bf16*)gate + (int64_t)t0 * g_st : nullptr,
+                                                            g_st, (__bf16*)out + (int64_t)t0 * H * d, nsplit, H, d);
+}
+
+// key splits of a portion whose last token sees max_keys keys: the causal lengths of the 16-token tiles differ
+// by a factor of two around their mean, so long portions are cut into more, shorter workgroups
+int talk_prefill_splits(int n, int max_keys) {
+  int ns = max_keys / 1024;
+  return ns < 1 ? 1 : (ns > 4 ? 4 : ns);
 }
 
 void talk_prefill(const float* q, const void* rows, int bs, const int32_t* bt, const int64_t* pos, int t0, int n,
-                  float scale, const float* talk, const void* gate, int64_t g_st, void* out, int H, int G, int d,
-                  hipStream_t st) {
+                  float scale, const float* talk, const void* gate, int64_t g_st, void* out, float* part, int nsplit,
+                  int H, int G, int d, hipStream_t st) {
   if (n <= 0 || !talk_prefill_fits(H, G, d)) return;
-#define BM_PF(D16, HW, NW) launch_prefill<D16, HW, NW>(q, rows, bs, bt, pos, t0, n, scale, talk, gate, g_st, out, G, st)
+#define BM_PF(D16, HW, NW) \
+  launch_prefill<D16, HW, NW>(q, rows, bs, bt, pos, t0, n, scale, talk, gate, g_st, out, G, part, nsplit, st)
   if (d == 64) {
     if (H == 4) BM_PF(4, 1, 4); else if (H == 8) BM_PF(4, 2, 4); else BM_PF(4, 2, 8);
   } else {

@@ -279,8 +279,8 @@ int64_t bm_talk_prefill_fits(int64_t H, int64_t G, int64_t d) {
 }
 
 void bm_talk_prefill(const Tensor& q, const Tensor& rows, const Tensor& table_row, const Tensor& pos, int64_t t0,
-                     int64_t n, double scale, const c10::optional<Tensor>& talk, const c10::optional<Tensor>& gate,
-                     int64_t G, Tensor& out) {
+                     int64_t n, int64_t max_keys, double scale, const c10::optional<Tensor>& talk,
+                     const c10::optional<Tensor>& gate, int64_t G, Tensor& out) {
   c10::DeviceGuard g(q.device());
   TORCH_CHECK(q.is_cuda() && q.dim() == 3 && q.scalar_type() == at::kFloat && q.is_contiguous(),
               "bm_talk_prefill: q f32 [T, H, d] contiguous");
@@ -307,9 +307,14 @@ void bm_talk_prefill(const Tensor& q, const Tensor& rows, const Tensor& table_ro
   TORCH_CHECK(out.is_cuda() && out.scalar_type() == at::kBFloat16 && out.is_contiguous() && out.dim() == 2 &&
                   out.size(0) == T && out.size(1) == H * d,
               "bm_talk_prefill: out bf16 [T, H d]");
+  TORCH_CHECK(max_keys >= n && max_keys <= table_row.numel() * rows.size(1),
+              "bm_talk_prefill: block table row narrower than the portion's context");
+  const int ns = illm::bm::talk_prefill_splits((int)n, (int)max_keys);
+  Tensor part;
+  if (ns > 1) part = at::empty({n, ns, H, d + 2}, q.options());
   illm::bm::talk_prefill(q.data_ptr<float>(), rows.data_ptr(), (int)rows.size(1), table_row.data_ptr<int32_t>(),
-                         pos.data_ptr<int64_t>(), (int)t0, (int)n, (float)scale, tp, gp, gst, out.data_ptr(), (int)H,
-                         (int)G, (int)d, stream());
+                         pos.data_ptr<int64_t>(), (int)t0, (int)n, (float)scale, tp, gp, gst, out.data_ptr(),
+                         ns > 1 ? part.data_ptr<float>() : nullptr, ns, (int)H, (int)G, (int)d, stream());
 }
 
 std::tuple<Tensor, Tensor> bm_talk_softmax(Tensor& sc, const Tensor& pos, int64_t H, double scale,
@@ -400,8 +405,8 @@ TORCH_LIBRARY_FRAGMENT(ipex_llm_amd, m) {
   m.def("bm_talk_attention(Tensor q, Tensor rows, Tensor block_tables, Tensor seq_of, Tensor pos, float scale, "
         "Tensor? talk, Tensor? gate, int G, int max_ctx, bool act_f32) -> Tensor");
   m.def("bm_talk_prefill_fits(int H, int G, int d) -> int");
-  m.def("bm_talk_prefill(Tensor q, Tensor rows, Tensor table_row, Tensor pos, int t0, int n, float scale, Tensor? talk, "
-        "Tensor? gate, int G, Tensor(a!) out) -> ()");
+  m.def("bm_talk_prefill(Tensor q, Tensor rows, Tensor table_row, Tensor pos, int t0, int n, int max_keys, float scale, "
+        "Tensor? talk, Tensor? gate, int G, Tensor(a!) out) -> ()");
   m.def("bm_talk_softmax(Tensor(a!) scores, Tensor pos, int H, float scale, Tensor? talk, bool act_f32) -> "
         "(Tensor, Tensor)");
   m.def("bm_moe_route(Tensor z, int top) -> (Tensor, Tensor)");

@@ -273,7 +273,7 @@ def _talk_attention_gpu(q, rows, block_tables, seq_of, pos, scale, talk, gate, G
     small, small_ctx, t0 = [], 1, 0
     for b, (n, L) in enumerate(zip(q_lens, ctx_lens)):
         if n >= min_q and mfma:
-            _ops().bm_talk_prefill(q, rows, block_tables[b], pos, t0, n, scale, talk, gate, G, out)
+            _ops().bm_talk_prefill(q, rows, block_tables[b], pos, t0, n, L, scale, talk, gate, G, out)
         elif n >= min_q:
             o = _talk_attention_gemm(q[t0:t0 + n], rows, block_tables[b], pos[t0:t0 + n], scale, talk, G, L, n)
             o = o.view(n, H * d)

@@ -311,7 +311,8 @@ def test_causal_edge(dev, edge):
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("H,G,d", [(8, 2, 64), (16, 4, 128), (4, 4, 64), (8, 1, 128), (16, 2, 64), (4, 1, 128), (6, 3, 40),
                                    (5, 5, 16), (12, 1, 20), (3, 3, 12)])
-def test_long_portion_paths_agree(H, G, d, dtype):
+@pytest.mark.parametrize("L,n", [(700, 633), (2300, 1101)])
+def test_long_portion_paths_agree(H, G, d, dtype, L, n):
     """portions past the thresholds take the matrix-core kernel (16-bit, its sizes) or library products with the
     fused mixing softmax between them; the same rows through the one-pass kernel give the same result.  The
     portion starts inside a page, ends inside a 16-token tile and shares the step with a decoded token."""
@@ -320,7 +321,9 @@ def test_long_portion_paths_agree(H, G, d, dtype):
     from ipex_llm_amd.ops import blockmix as BM
     dev = torch.device("cuda")
     g = torch.Generator().manual_seed(d)
-    L, n = 700, 633                                   # the portion starts 67 tokens into the sequence
+    if L > 1000 and (dtype == torch.float32 or d % 64):
+        pytest.skip("the long case is for the matrix-core kernel's key splits")
+    # the portion starts inside a page, 67 (1199) tokens into the sequence; past 2048 keys the kernel splits them
     k, v = torch.randn(L, G, d, generator=g).to(dtype), torch.randn(L, G, d, generator=g).to(dtype)
     q = torch.randn(n + 1, H, d, generator=g)
     talk = torch.eye(H) + 0.3 * torch.randn(H, H, generator=g)
@@ -336,7 +339,7 @@ def test_long_portion_paths_agree(H, G, d, dtype):
     tol = 2e-5 if dtype == torch.float32 else 2e-2
     old = BM.GEMM_MIN_Q, BM.MFMA_MIN_Q
     try:
-        for gemm_min, mfma_min in (old, (128, 0), (1 << 30, 0)):
+        for gemm_min, mfma_min in ((old,) if L > 1000 else (old, (128, 0), (1 << 30, 0))):
             BM.GEMM_MIN_Q, BM.MFMA_MIN_Q = gemm_min, mfma_min
             got = BM.talk_attention(*args).cpu().double()
             assert (got - want).abs().max() < tol, (gemm_min, mfma_min)
