@@ -48,9 +48,9 @@ __device__ __forceinline__ void wave_sync() {
 }
 
 // ------------------------------------------------------------------ norm + rotary + cache append
-// one block per token, one wave per head in turn (query heads, then key heads); buf: 4 x d floats
+// one block per token, one wave per head in turn (query heads, then key heads); buf: (waves) x d floats
 template <typename E>
-__global__ void __launch_bounds__(256) qk_norm_rope_store_k(const E* __restrict__ q, int64_t q_ld, const E* __restrict__ k,
+__global__ void __launch_bounds__(1024) qk_norm_rope_store_k(const E* __restrict__ q, int64_t q_ld, const E* __restrict__ k,
                                                            int64_t k_ld, const E* __restrict__ qn, const E* __restrict__ kn,
                                                            float eps, const float* __restrict__ table, int max_pos,
                                                            int dims, const int64_t* __restrict__ pos,
@@ -67,7 +67,8 @@ __global__ void __launch_bounds__(256) qk_norm_rope_store_k(const E* __restrict_
   const int half = dims >> 1;
   const int64_t slot = slots[t];
   const bool store = slot >= 0 && slot < num_rows;
-  for (int hh = wv; hh < H + G; hh += 4) {
+  const int nwv = blockDim.x >> 6;
+  for (int hh = wv; hh < H + G; hh += nwv) {
     const bool isq = hh < H;
     const E* src = isq ? q + t * q_ld + (int64_t)hh * d : k + t * k_ld + (int64_t)(hh - H) * d;
     const E* nw = isq ? qn : kn;
@@ -760,13 +761,16 @@ void qk_norm_rope_store(bool bf16, const void* q, int64_t q_ld, const void* k, i
                         const int64_t* slots, void* rows, int64_t num_rows, float* qo, int T, int H, int G, int d,
                         hipStream_t st) {
   if (T <= 0) return;
-  const size_t lds = (size_t)4 * d * sizeof(float);
+  int nwv = H + G >= 16 ? 16 : H + G;               // few rows: a wave per head, within 48 KB of LDS
+  if (T > 64 && nwv > 4) nwv = 4;
+  if (nwv * d > 12288) nwv = 12288 / d < 1 ? 1 : 12288 / d;
+  const size_t lds = (size_t)nwv * d * sizeof(float);
   if (bf16)
-    qk_norm_rope_store_k<__bf16><<<T, 256, lds, st>>>((const __bf16*)q, q_ld, (const __bf16*)k, k_ld, (const __bf16*)qn,
+    qk_norm_rope_store_k<__bf16><<<T, 64 * nwv, lds, st>>>((const __bf16*)q, q_ld, (const __bf16*)k, k_ld, (const __bf16*)qn,
                                                       (const __bf16*)kn, eps, table, max_pos, dims, pos, slots,
                                                       (__bf16*)rows, num_rows, qo, H, G, d);
   else
-    qk_norm_rope_store_k<float><<<T, 256, lds, st>>>((const float*)q, q_ld, (const float*)k, k_ld, (const float*)qn,
+    qk_norm_rope_store_k<float><<<T, 64 * nwv, lds, st>>>((const float*)q, q_ld, (const float*)k, k_ld, (const float*)qn,
                                                      (const float*)kn, eps, table, max_pos, dims, pos, slots,
                                                      (float*)rows, num_rows, qo, H, G, d);
 }

@@ -38,7 +38,7 @@ __device__ __forceinline__ float block_sum(float v, float* red) {
 }
 
 template <typename E>
-__global__ void __launch_bounds__(256) rms_norm_rows_k(const float* __restrict__ x, const E* __restrict__ w, int nw,
+__global__ void __launch_bounds__(1024) rms_norm_rows_k(const float* __restrict__ x, const E* __restrict__ w, int nw,
                                                       float* __restrict__ h, E* __restrict__ ha, int W, float eps) {
   __shared__ float red[16];
   const int64_t t = blockIdx.x;
@@ -55,7 +55,7 @@ __global__ void __launch_bounds__(256) rms_norm_rows_k(const float* __restrict__
 }
 
 template <typename E>
-__global__ void __launch_bounds__(256) add_rms_norm_k(float* __restrict__ x, const E* __restrict__ y,
+__global__ void __launch_bounds__(1024) add_rms_norm_k(float* __restrict__ x, const E* __restrict__ y,
                                                      const E* __restrict__ w, E* __restrict__ xa, int W, float eps) {
   __shared__ float red[16];
   const int64_t t = blockIdx.x;
@@ -154,7 +154,7 @@ __global__ void __launch_bounds__(256) canon_state_k(const float* __restrict__ h
 // is the only reader of its sequence's state and advances it itself; otherwise canon_state_k follows.
 constexpr int kMaxTaps = 16;
 template <typename E>
-__global__ void __launch_bounds__(256) norm_canon_k(const float* __restrict__ x, const E* __restrict__ g, int ng,
+__global__ void __launch_bounds__(1024) norm_canon_k(const float* __restrict__ x, const E* __restrict__ g, int ng,
                                                    float eps, const float* __restrict__ w, int taps,
                                                    float* __restrict__ state, const int32_t* __restrict__ cu,
                                                    const int32_t* __restrict__ seq_of, const int32_t* __restrict__ slots,
@@ -241,6 +241,12 @@ __global__ void __launch_bounds__(256) side_gate_k(const E* __restrict__ z, cons
   }
 }
 
+// threads of a one-row-per-block kernel.  Few rows (decode): a thread per channel or two, since a thread's loads
+// are dependent and the launch is latency-bound; many rows: 256, several blocks per CU
+int row_threads(int W, int T) {
+  if (T > 64) return 256;
+  return W >= 1024 ? 1024 : (W <= 64 ? 64 : (W + 63) / 64 * 64);
+}
 int grid_for(int64_t n) { return (int)((n + 255) / 256 < 1 ? 1 : ((n + 255) / 256 > 65535 ? 65535 : (n + 255) / 256)); }
 
 }  // namespace
@@ -248,14 +254,14 @@ int grid_for(int64_t n) { return (int)((n + 255) / 256 < 1 ? 1 : ((n + 255) / 25
 void rms_norm_rows(bool bf16, const float* x, const void* w, int nw, float* h, void* ha, int T, int W, float eps,
                    hipStream_t st) {
   if (T <= 0) return;
-  if (bf16) rms_norm_rows_k<__bf16><<<T, 256, 0, st>>>(x, (const __bf16*)w, nw, h, (__bf16*)ha, W, eps);
-  else rms_norm_rows_k<float><<<T, 256, 0, st>>>(x, (const float*)w, nw, h, nullptr, W, eps);
+  if (bf16) rms_norm_rows_k<__bf16><<<T, row_threads(W, T), 0, st>>>(x, (const __bf16*)w, nw, h, (__bf16*)ha, W, eps);
+  else rms_norm_rows_k<float><<<T, row_threads(W, T), 0, st>>>(x, (const float*)w, nw, h, nullptr, W, eps);
 }
 
 void add_rms_norm(bool bf16, float* x, const void* y, const void* w, void* xa, int T, int W, float eps, hipStream_t st) {
   if (T <= 0) return;
-  if (bf16) add_rms_norm_k<__bf16><<<T, 256, 0, st>>>(x, (const __bf16*)y, (const __bf16*)w, (__bf16*)xa, W, eps);
-  else add_rms_norm_k<float><<<T, 256, 0, st>>>(x, (const float*)y, (const float*)w, nullptr, W, eps);
+  if (bf16) add_rms_norm_k<__bf16><<<T, row_threads(W, T), 0, st>>>(x, (const __bf16*)y, (const __bf16*)w, (__bf16*)xa, W, eps);
+  else add_rms_norm_k<float><<<T, row_threads(W, T), 0, st>>>(x, (const float*)y, (const float*)w, nullptr, W, eps);
 }
 
 void residual_add_scaled(bool bf16, float* x, const void* y1, const float* s1, const void* y2, bool y2_f32,
@@ -284,10 +290,10 @@ void norm_canon(bool bf16, const float* x, const void* g, int ng, float eps, con
                 void* out, int T, int B, int W, bool single, hipStream_t st) {
   if (T <= 0) return;
   if (bf16)
-    norm_canon_k<__bf16><<<T, 256, 0, st>>>(x, (const __bf16*)g, ng, eps, w, taps, state, cu, seq_of, slots, pos, h,
+    norm_canon_k<__bf16><<<T, row_threads(W, T), 0, st>>>(x, (const __bf16*)g, ng, eps, w, taps, state, cu, seq_of, slots, pos, h,
                                             (__bf16*)ha, (__bf16*)out, W, single ? 1 : 0);
   else
-    norm_canon_k<float><<<T, 256, 0, st>>>(x, (const float*)g, ng, eps, w, taps, state, cu, seq_of, slots, pos, h,
+    norm_canon_k<float><<<T, row_threads(W, T), 0, st>>>(x, (const float*)g, ng, eps, w, taps, state, cu, seq_of, slots, pos, h,
                                            nullptr, (float*)out, W, single ? 1 : 0);
   if (!single) canon_state_k<<<B, 256, 0, st>>>(h, taps, state, cu, slots, pos, W);
 }
