@@ -651,3 +651,26 @@ def test_experts_bf16(dev, T, E, top, Wd, ff):
         for j in range(top):
             want[t] += O.expert(W64, f"e{int(idx[t, j])}.", float(w[t, j]) * h[t].double(), 1.5)
     assert (got - want).abs().max() < 0.03 * float(want.abs().max())
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_matrix_core_sizes_model(dev, dtype):
+    """a model whose head sizes and head counts fall into the matrix-core kernels' set (64-wide heads; 8, 4 and
+    16 heads over 4, 1 and 2 key / value heads): portions past and below the kernels' thresholds beside decoded
+    tokens of a second sequence, then decoding"""
+    cfg = O.config([O.attn_layer(heads=8, kv_heads=4, dim=64, scaling=YARN, mlp=O.moe(4, 2, 32, 2.0, 32, 1.0)),
+                    O.attn_layer(heads=4, kv_heads=1, dim=64, dims=32, mlp=O.dense(96)),
+                    O.attn_layer(heads=16, kv_heads=2, dim=64, base=500.0, mlp=None)], width=64, taps=3, side=8)
+    W = O.random_weights(cfg, 31)
+    if dtype == torch.bfloat16:                      # 16-bit runs: prompts far from close router calls
+        seeds = sorted(range(40), key=lambda s: -O.router_margin(cfg, W, O.random_tokens(cfg, 40, s)))
+        P = {"a": O.random_tokens(cfg, 40, seeds[0]), "b": O.random_tokens(cfg, 40, seeds[1])}
+        schedule = [[("a", 35), ("b", 1)], [("a", 2), ("b", 33)], [("a", 1), ("b", 1)], [("a", 1), ("b", 1)],
+                    [("a", 1), ("b", 4)]]
+    else:
+        P = {"a": clear_tokens(cfg, W, 140, 1), "b": clear_tokens(cfg, W, 40, 2)}
+        schedule = [[("a", 70), ("b", 1)], [("a", 3), ("b", 33)], [("a", 40), ("b", 1)]] + [[("a", 1), ("b", 1)]] * 5 + \
+            [[("a", 22)]]
+    got = replay(engine(cfg, W, dev, dtype), P, schedule)
+    for name, toks in P.items():
+        assert rel_err(got[name], O.forward(cfg, W, toks)) < TOL[dtype], name
