@@ -269,7 +269,10 @@ class GroupedAttention(nn.Module):
     def ensure_table(self, max_pos: int):
         if self.table is None or self.table.shape[0] < max_pos or self.table.device != self.w_o.device:
             n = max(256, 1 << (max_pos - 1).bit_length())
-            self.table = SM.rope_table(n, self.s.rot.dims, self.s.rot.base, self.s.rot.scaling).to(self.w_o.device)
+            if self.s.rot is None or self.s.rot.dims == 0:     # no rotation: one pair turned by the angle 0
+                self.table = torch.tensor([1.0, 0.0]).repeat(n, 1, 1).contiguous().to(self.w_o.device)
+            else:
+                self.table = SM.rope_table(n, self.s.rot.dims, self.s.rot.base, self.s.rot.scaling).to(self.w_o.device)
         return self.table
 
     def forward(self, xa, pos, slots, meta: AttnMeta, cache, li: int, eps: float):

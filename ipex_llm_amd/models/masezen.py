@@ -36,7 +36,7 @@ def spec_from_config(cfg: dict) -> HybridSpec:
         m, kind = L["mixer"], L["type"]
         if kind != "attention":
             raise ValueError(f"layer {i}: unknown mixer type {kind!r}")
-        rot = m["rot"]
+        rot = m.get("rot") or {"dims": 0, "base": 10000.0}
         if int(m.get("vdim", m["dim"])) != int(m["dim"]):
             raise ValueError(f"layer {i}: the values are the keys, so vdim must equal dim")
         mixer = GroupedAttentionSpec(heads=int(m["heads"]), kv_heads=int(m["kv_heads"]), dim=int(m["dim"]),

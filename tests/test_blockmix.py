@@ -422,6 +422,8 @@ LAYER_CASES = [
     # head sizes that are no multiple of 8 and more than 8 query heads per key / value head: no one-pass kernel
     ([O.attn_layer(heads=5, kv_heads=5, dim=12, dims=6, mlp=O.moe(3, 2, 12, 2.0, 20, 1.0))], dict(width=20, taps=3, side=2)),
     ([O.attn_layer(heads=12, kv_heads=1, dim=20, scaling=YARN, mlp=O.dense(36))], dict(width=36, taps=2, side=0)),
+    # no rotated part at all
+    ([O.attn_layer(heads=2, kv_heads=1, dim=16, dims=0, mlp=O.dense(24))], dict(width=24, taps=3, side=4)),
 ]
 
 
